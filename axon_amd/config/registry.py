@@ -28,10 +28,13 @@ def known_architectures():
 
 
 def architecture_of(cfg: Dict[str, Any]) -> str:
-    """`model_type` decides if it is a known one; else `architectures[0]`."""
+    """`model_type` decides if it is a known one; else `architectures[0]`, or the single name
+    a config.json gives as `architecture`."""
     mt = cfg.get("model_type") or ""
     archs = cfg.get("architectures") or []
     hf = archs[0] if isinstance(archs, list) and archs and isinstance(archs[0], str) else ""
+    if not hf and isinstance(cfg.get("architecture"), str):
+        hf = cfg["architecture"]
     if isinstance(mt, str) and mt in _MODEL_TYPES:
         return _MODEL_TYPES[mt]
     if hf in _ARCHITECTURES:

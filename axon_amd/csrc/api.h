@@ -194,6 +194,84 @@ int axk_topk(float* logits, int logits_stride, const int32_t* recent, int recent
 int axk_fill_i32(int32_t* dst, int32_t value, int n, void* stream);
 int axk_fill_f32(float* dst, float value, int n, void* stream);
 
+// axk_embed with every value multiplied by `scale` (32-bit) on the way.
+int axk_embed_scaled(const int32_t* tokens, const void* table, int packed, float* x, int n_tokens, int dim, int vocab,
+                     float scale, void* stream);
+
+// A norm on a sublayer's output: x[r, :] += mult * ((y[r, :] * inv_rms(y[r, :])) * gain); `rounded`
+// (elem [n_rows, dim], or null) also gets the new x in the compute dtype.
+int axk_norm_add(const float* y, const void* gain, int gain_is_f32, float eps, float mult, float* x, void* rounded,
+                 int n_rows, int dim, void* stream);
+// out[i] = x[i] in the compute dtype.
+int axk_round_rows(const float* x, void* out, long n, void* stream);
+// In place on elem values; kind 0: the tanh form of GELU.
+int axk_activation(void* v, long n, int kind, void* stream);
+// out[t, f] = g sigmoid(alpha g) (u + 1), g = min(gate_up[t, f], limit), u = clamp(gate_up[t, F + f], -limit, limit).
+int axk_clamped_glu(const void* gate_up, void* out, int n_tokens, int n_ffn, float limit, float alpha, void* stream);
+
+// Grouped products (csrc/grouped_gemm.hip):
+//   out[orow(r), g ogs + n] = epilogue(sum_k X[xrow(r), g xgs + k] W[g][n][k] + bias[g][n]),
+// W elem [groups][n (2 n with glu)][k].  tiles == null: every row r < m meets every group
+// (block-diagonal; x_rows and out_rows must be null).  tiles [.][3] = (group, first listed row,
+// count <= 16) with *n_tiles of them on the device (max_tiles: the most there can be): the rows
+// listed, x_rows / out_rows naming the row of X each reads and the row of out it writes (null:
+// the listed row itself).  glu: g = min(gate, limit), u = clamp(up, -limit, limit), out = g
+// sigmoid(alpha g) (u + 1).  gate (float32, rows gate_row_stride apart): out is multiplied by
+// sigmoid(gate[orow, g ogs + n]).  Strides count elements.  An output's chain over k depends on
+// k, the strides' alignment and the build alone (axk_grouped_gemm_uses_mfma says which chain).
+int axk_grouped_gemm_uses_mfma(int k, int x_is_f32, long x_row_stride, long x_group_stride);
+int axk_grouped_gemm(const void* x, int x_is_f32, long x_row_stride, long x_group_stride, const int32_t* x_rows,
+                     const void* w, const void* bias, int bias_is_f32, void* out, int out_is_f32, long out_row_stride,
+                     long out_group_stride, const int32_t* out_rows, const float* gate, long gate_row_stride, int glu,
+                     float glu_limit, float glu_alpha, const int32_t* tiles, const int32_t* n_tiles, int max_tiles, int m,
+                     int n, int k, int groups, void* stream);
+
+// Routing (csrc/moe.hip).  axk_route_topk: for each token the `top` largest of its n_experts
+// logits (the largest first; of equal ones the lower expert) and the softmax over these.
+// axk_route_sort: the pairs p = t top + k in expert order (sorted, and each one's token in
+// sorted_tokens) and the tiles of the grouped product, at most axk_route_max_tiles of them.
+// axk_route_combine: y[t, :] (+)= sum_k weights[t, k] rows[t top + k, :], k ascending.
+int axk_route_topk(const float* logits, int n_tokens, int n_experts, int top, int32_t* experts, float* weights, void* stream);
+int axk_route_max_tiles(int n_pairs, int n_experts);
+int axk_route_sort(const int32_t* experts, int n_pairs, int n_experts, int top, int32_t* sorted, int32_t* sorted_tokens,
+                   int32_t* tiles, int32_t* n_tiles, void* stream);
+int axk_route_combine(const float* rows, const float* weights, float* y, int n_tokens, int top, int width, int accumulate,
+                      void* stream);
+
+// A short causal convolution per channel and a gated linear recurrence (csrc/recurrent.hip).  A
+// request's state row (float32, rows state_stride apart) is [channels] of recurrent state, then
+// [taps - 1][channels] of the convolution's last inputs, oldest first; zeros for a new request.
+// axk_causal_conv: u[t, c] = bias[c] + sum_k w[c, k] in(t - (taps - 1 - k)), inputs before the
+// step from the state (state_offset: where the kept inputs start in a row).  Reads the state only.
+// axk_gated_scan: per request of the step (spans [n][3] = (slot, first token, tokens); null: each
+// token a request of its own in slot seq_rows[t]) and channel, over its tokens in order:
+// r = sigmoid(gates r), i = sigmoid(gates i), a = exp(-decay r softplus(lam)),
+// S = a S + sqrt(1 - a^2) (i u), out = S gelu(y); then the state row is brought up to date
+// (S, and the convolution's inputs from x).  gates [T, channels / block_width, 2 block_width].
+int axk_causal_conv(const void* x, long x_stride, const void* w, const void* bias, int bias_is_f32, const float* state,
+                    long state_stride, int state_offset, const int32_t* seq_rows, float* u, int n_tokens, int channels,
+                    int taps, void* stream);
+int axk_gated_scan(const float* gates, const float* u, const void* y, long y_stride, const void* x, long x_stride,
+                   const void* lam, int lam_is_f32, float decay, float* state, long state_stride, const int32_t* spans,
+                   int n_spans, const int32_t* seq_rows, void* out, int channels, int block_width, int taps, void* stream);
+
+// Attention over a latent cache (csrc/latent_attention.hip); a page is [page_size][rank + rot] elem.
+// axk_latent_prepare: from the float32 rows of the down projections, the normed query latent
+// (cq elem [T, q_rank]; q_rank 0: none) and, with write_kv, the normed key/value latent and the
+// rotated shared key part into the request's page.  axk_latent_query_rope: the rotated part of
+// every head's query into q_full [T, heads, rank + rot] (places rank ..).  axk_latent_attention:
+// o_lat [T, heads, rank] = softmax over lo ..= pos of (q_full . page row) scale, times the rows'
+// first `rank` places; lo = window > 0 ? max(0, pos + 1 - window) : 0.
+int axk_latent_prepare(const float* fused, long stride, int q_at, int q_rank, int kv_at, int rank, int rot, int rot_dims,
+                       const void* q_gain, int q_gain_is_f32, const void* kv_gain, int kv_gain_is_f32, float eps,
+                       const float* table, const int32_t* positions, const int32_t* seq_rows, const int32_t* block_table,
+                       int table_stride, void* cache, int page_size, void* cq, int n_tokens, int write_kv, void* stream);
+int axk_latent_query_rope(const float* q, int dim, int rot, int rot_dims, const float* table, float* q_full, int rank,
+                          int heads, int n_tokens, void* stream);
+int axk_latent_attention(const float* q_full, const void* cache, const int32_t* block_table, int table_stride,
+                         const int32_t* positions, const int32_t* seq_rows, float* o_lat, int n_tokens, int heads, int rank,
+                         int rot, int page_size, int window, float scale, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

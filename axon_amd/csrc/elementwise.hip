@@ -11,28 +11,34 @@
 // A tied head's matrix is kept packed for the products (see axk_pack_matrix): element (row, i) is
 // then at ((row / 16 * dim / 32 + i / 32) * 64 + row % 16 + 16 (i % 32 / 8)) * 8 + i % 8.
 __global__ void embed_kernel(const int32_t* __restrict__ tokens, const elem_t* __restrict__ table, int packed,
-                             float* __restrict__ x, int dim) {
+                             float* __restrict__ x, int dim, float scale) {
   const int t = blockIdx.x;
   const int token = tokens[t];
   float* dst = x + (size_t)t * dim;
   if (packed) {
     const elem_t* tile = table + (size_t)(token / 16) * (dim / 32) * 512 + (token % 16) * 8;
     for (int i = threadIdx.x; i < dim; i += blockDim.x)
-      dst[i] = to_float(tile[(size_t)(i / 32) * 512 + ((i % 32) / 8) * 128 + i % 8]);
+      dst[i] = to_float(tile[(size_t)(i / 32) * 512 + ((i % 32) / 8) * 128 + i % 8]) * scale;
     return;
   }
   const elem_t* row = table + (size_t)token * dim;
-  for (int i = threadIdx.x; i < dim; i += blockDim.x) dst[i] = to_float(row[i]);
+  for (int i = threadIdx.x; i < dim; i += blockDim.x) dst[i] = to_float(row[i]) * scale;
 }
 
-extern "C" int axk_embed(const int32_t* tokens, const void* table, int packed, float* x, int n_tokens, int dim,
-                         int vocab, void* stream) {
+extern "C" int axk_embed_scaled(const int32_t* tokens, const void* table, int packed, float* x, int n_tokens, int dim,
+                                int vocab, float scale, void* stream) {
   AXK_REQUIRE(n_tokens >= 0 && dim > 0 && vocab > 0, "embed: bad sizes T=%d dim=%d vocab=%d", n_tokens, dim, vocab);
   AXK_REQUIRE(!packed || dim % 32 == 0, "embed: a packed table has rows of whole blocks of 32, not %d", dim);
   if (n_tokens == 0) return 0;
-  embed_kernel<<<n_tokens, 256, 0, (hipStream_t)stream>>>(tokens, (const elem_t*)table, packed, x, dim);
+  embed_kernel<<<n_tokens, 256, 0, (hipStream_t)stream>>>(tokens, (const elem_t*)table, packed, x, dim, scale);
   AXK_LAUNCH_CHECK("embed");
   return 0;
+}
+
+// a factor of 1 leaves the widened values as they are
+extern "C" int axk_embed(const int32_t* tokens, const void* table, int packed, float* x, int n_tokens, int dim,
+                         int vocab, void* stream) {
+  return axk_embed_scaled(tokens, table, packed, x, n_tokens, dim, vocab, 1.0f, stream);
 }
 
 // ---------------------------------------------------------------------------- RMSNorm
@@ -247,6 +253,87 @@ extern "C" int axk_swiglu(const void* gate_up, void* out, int n_tokens, int n_ff
   dim3 grid(ceil_div(n_ffn, 256), n_tokens);
   swiglu_kernel<<<grid, 256, 0, (hipStream_t)stream>>>((const elem_t*)gate_up, (elem_t*)out, n_ffn);
   AXK_LAUNCH_CHECK("swiglu");
+  return 0;
+}
+
+// ---------------------------------------------------------------------------- a norm on a sublayer's output
+// x[r, :] += mult * ((y[r, :] * inv_rms(y[r, :])) * gain), and rounded[r, :] = x[r, :] in the compute
+// dtype if asked for (what the next sublayer's products read).  The sum of squares as in rmsnorm_kernel.
+__global__ void __launch_bounds__(NORM_THREADS)
+norm_add_kernel(const float* __restrict__ y, const void* __restrict__ gain, int gain_is_f32, float eps, float mult,
+                float* __restrict__ x, elem_t* __restrict__ rounded, int dim) {
+  __shared__ float partial[NORM_THREADS / AXON_WAVE];
+  const int r = blockIdx.x;
+  const float* src = y + (size_t)r * dim;
+  float ss = 0.0f;
+  for (int i = threadIdx.x; i < dim; i += NORM_THREADS) ss = fmaf(src[i], src[i], ss);
+  const float inv = 1.0f / sqrtf(block_sum_256(ss, partial) / (float)dim + eps);
+  float* dst = x + (size_t)r * dim;
+  for (int i = threadIdx.x; i < dim; i += NORM_THREADS) {
+    const float v = dst[i] + mult * ((src[i] * inv) * load_vec(gain, gain_is_f32, i));
+    dst[i] = v;
+    if (rounded) rounded[(size_t)r * dim + i] = from_float(v);
+  }
+}
+
+extern "C" int axk_norm_add(const float* y, const void* gain, int gain_is_f32, float eps, float mult, float* x, void* rounded,
+                            int n_rows, int dim, void* stream) {
+  AXK_REQUIRE(n_rows >= 0 && dim > 0, "norm_add: bad sizes rows=%d dim=%d", n_rows, dim);
+  if (n_rows == 0) return 0;
+  norm_add_kernel<<<n_rows, NORM_THREADS, 0, (hipStream_t)stream>>>(y, gain, gain_is_f32, eps, mult, x, (elem_t*)rounded, dim);
+  AXK_LAUNCH_CHECK("norm_add");
+  return 0;
+}
+
+// out[i] = x[i] in the compute dtype.
+__global__ void round_rows_kernel(const float* __restrict__ x, elem_t* __restrict__ out, long n) {
+  const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) out[i] = from_float(x[i]);
+}
+
+extern "C" int axk_round_rows(const float* x, void* out, long n, void* stream) {
+  if (n <= 0) return 0;
+  round_rows_kernel<<<(unsigned)((n + 255) / 256), 256, 0, (hipStream_t)stream>>>(x, (elem_t*)out, n);
+  AXK_LAUNCH_CHECK("round_rows");
+  return 0;
+}
+
+// ---------------------------------------------------------------------------- activations
+// kind 0: the tanh form of GELU, 0.5 z (1 + tanh(sqrt(2 / pi) (z + 0.044715 z^3))), in place.
+__global__ void activation_kernel(elem_t* __restrict__ v, long n, int kind) {
+  const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  const float z = to_float(v[i]);
+  const float inner = 0.7978845608028654f * (z + 0.044715f * ((z * z) * z));
+  v[i] = from_float((0.5f * z) * (1.0f + tanhf(inner)));
+}
+
+extern "C" int axk_activation(void* v, long n, int kind, void* stream) {
+  AXK_REQUIRE(kind == 0, "activation: kind %d is not known (0: gelu, tanh form)", kind);
+  if (n <= 0) return 0;
+  activation_kernel<<<(unsigned)((n + 255) / 256), 256, 0, (hipStream_t)stream>>>((elem_t*)v, n, kind);
+  AXK_LAUNCH_CHECK("activation");
+  return 0;
+}
+
+// out[t, f] = g sigmoid(alpha g) (u + 1) with g = min(gu[t, f], limit), u = clamp(gu[t, F + f], -limit, limit).
+__global__ void clamped_glu_kernel(const elem_t* __restrict__ gate_up, elem_t* __restrict__ out, int n_ffn, float limit,
+                                   float alpha) {
+  const int t = blockIdx.y;
+  const int f = blockIdx.x * blockDim.x + threadIdx.x;
+  if (f >= n_ffn) return;
+  const elem_t* row = gate_up + (size_t)t * 2 * n_ffn;
+  const float g = fminf(to_float(row[f]), limit);
+  const float u = fminf(fmaxf(to_float(row[n_ffn + f]), -limit), limit);
+  out[(size_t)t * n_ffn + f] = from_float((g * (1.0f / (1.0f + expf(-(alpha * g))))) * (u + 1.0f));
+}
+
+extern "C" int axk_clamped_glu(const void* gate_up, void* out, int n_tokens, int n_ffn, float limit, float alpha, void* stream) {
+  AXK_REQUIRE(n_tokens >= 0 && n_ffn > 0 && n_tokens <= 65535, "clamped_glu: bad sizes T=%d ffn=%d", n_tokens, n_ffn);
+  if (n_tokens == 0) return 0;
+  dim3 grid(ceil_div(n_ffn, 256), n_tokens);
+  clamped_glu_kernel<<<grid, 256, 0, (hipStream_t)stream>>>((const elem_t*)gate_up, (elem_t*)out, n_ffn, limit, alpha);
+  AXK_LAUNCH_CHECK("clamped_glu");
   return 0;
 }
 

@@ -1,0 +1,247 @@
+// Grouped products: many small matrices, each applied to its own rows or its own columns.
+//
+//   out[orow(r), g ogs + n] = epilogue( sum_k X[xrow(r), g xgs + k] W[g][n][k] + bias[g][n] )
+//
+// Two ways of saying which rows meet which matrix:
+//   * block-diagonal (tiles == null): every row r < M goes through every group g < G, group g
+//     reading its own slice of the row's columns (a recurrent layer's gates per block of channels,
+//     a per-head projection of an attention layer);
+//   * routed (tiles given, on the device): the rows are listed per group in tiles of up to 16
+//     (group, first row, count); xrow / orow name the row of X a listed row reads and the row of
+//     out it writes (a mixture of experts: rows are (token, chosen expert) pairs in expert order).
+//     The grid is launched for the most tiles there can be; blocks beyond *n_tiles leave at once.
+//
+// Epilogues: bias; a gated linear unit with clamps (W holds 2 N rows a group, gate rows then up
+// rows: g = min(gate, limit), u = clamp(up, -limit, limit), out = g sigmoid(alpha g) (u + 1));
+// a multiplication by sigmoid(gate[orow, g ogs + n]); out in float32 or in the compute dtype.
+//
+// The K-reduction of one output is one chain in ascending k that depends on K and the build alone
+// (32-bit FMA, or 16x16x32 MFMAs where the bfloat16 build can use them: K a multiple of 32 and
+// 16-byte aligned rows), never on which other rows share the tile.
+#include "api.h"
+#include "common.h"
+#include "instances.h"
+
+namespace {
+
+struct GroupedArgs {
+  const void* x; int x_is_f32; long x_row_stride; long x_group_stride; const int32_t* x_rows;
+  const elem_t* w; const void* bias; int bias_is_f32;
+  void* out; int out_is_f32; long out_row_stride; long out_group_stride; const int32_t* out_rows;
+  const float* gate; long gate_row_stride;
+  int glu; float glu_limit; float glu_alpha;
+  const int32_t* tiles; const int32_t* n_tiles;
+  int M, N, K, G;
+};
+
+#define GG_ROWS 16
+#define GG_COLS 64
+#define GG_BK 32
+
+__device__ inline float gg_load_x(const GroupedArgs& a, long at) {
+  return a.x_is_f32 ? ((const float*)a.x)[at] : to_float(((const elem_t*)a.x)[at]);
+}
+
+__device__ inline float clamped_glu(float gate, float up, float limit, float alpha) {
+  const float g = fminf(gate, limit);
+  const float u = fminf(fmaxf(up, -limit), limit);
+  return (g * (1.0f / (1.0f + expf(-(alpha * g))))) * (u + 1.0f);
+}
+
+__device__ inline void gg_store(const GroupedArgs& a, int g, int orow, int n, float v, float up) {
+  if (a.bias) {
+    const int per = a.glu ? 2 * a.N : a.N;
+    v += load_vec(a.bias, a.bias_is_f32, g * per + n);
+    if (a.glu) up += load_vec(a.bias, a.bias_is_f32, g * per + a.N + n);
+  }
+  if (a.glu) v = clamped_glu(v, up, a.glu_limit, a.glu_alpha);
+  const long col = (long)g * a.out_group_stride + n;
+  if (a.gate) v = v * (1.0f / (1.0f + expf(-a.gate[(long)orow * a.gate_row_stride + col])));
+  const long at = (long)orow * a.out_row_stride + col;
+  if (a.out_is_f32) ((float*)a.out)[at] = v;
+  else ((elem_t*)a.out)[at] = from_float(v);
+}
+
+// which rows and which group this block works on; false: nothing
+__device__ inline bool gg_tile(const GroupedArgs& a, int& g, int& first, int& count) {
+  if (a.tiles) {
+    if ((int)blockIdx.x >= *a.n_tiles) return false;
+    g = a.tiles[3 * blockIdx.x];
+    first = a.tiles[3 * blockIdx.x + 1];
+    count = a.tiles[3 * blockIdx.x + 2];
+  } else {
+    g = blockIdx.z;
+    first = blockIdx.x * GG_ROWS;
+    count = min(GG_ROWS, a.M - first);
+  }
+  return count > 0;
+}
+
+// 16 rows x 64 columns a block of 256 threads: thread (ty, tx) owns rows 4 ty .. 4 ty + 3 of column tx.
+template <bool GLU>
+__global__ void __launch_bounds__(256) grouped_gemm_fma_kernel(GroupedArgs a) {
+  __shared__ float xs[GG_ROWS][GG_BK + 1];
+  __shared__ float ws[GG_COLS][GG_BK + 1];
+  __shared__ float us[GLU ? GG_COLS : 1][GG_BK + 1];
+  __shared__ int xrow[GG_ROWS], orow[GG_ROWS];
+  int g, first, count;
+  if (!gg_tile(a, g, first, count)) return;
+  const int tid = threadIdx.x, tx = tid & 63, ty = tid >> 6;
+  const int n0 = blockIdx.y * GG_COLS;
+  if (tid < GG_ROWS) {
+    const int r = first + min(tid, count - 1);
+    xrow[tid] = a.x_rows ? a.x_rows[r] : r;
+    orow[tid] = a.out_rows ? a.out_rows[r] : r;
+  }
+  __syncthreads();
+  const int w_rows = GLU ? 2 * a.N : a.N;
+  const elem_t* wg = a.w + (long)g * w_rows * a.K;
+  float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f}, acc_up[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+  for (int k0 = 0; k0 < a.K; k0 += GG_BK) {
+    for (int i = tid; i < GG_ROWS * GG_BK; i += 256) {
+      const int r = i / GG_BK, kk = i % GG_BK;
+      xs[r][kk] = (r < count && k0 + kk < a.K)
+                      ? gg_load_x(a, (long)xrow[r] * a.x_row_stride + (long)g * a.x_group_stride + k0 + kk) : 0.0f;
+    }
+    for (int i = tid; i < GG_COLS * GG_BK; i += 256) {
+      const int c = i / GG_BK, kk = i % GG_BK;
+      const bool ok = n0 + c < a.N && k0 + kk < a.K;
+      ws[c][kk] = ok ? to_float(wg[(long)(n0 + c) * a.K + k0 + kk]) : 0.0f;
+      if (GLU) us[c][kk] = ok ? to_float(wg[(long)(a.N + n0 + c) * a.K + k0 + kk]) : 0.0f;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int kk = 0; kk < GG_BK; ++kk) {
+      const float b = ws[tx][kk];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) acc[i] = fmaf(xs[ty * 4 + i][kk], b, acc[i]);
+      if (GLU) {
+        const float bu = us[tx][kk];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) acc_up[i] = fmaf(xs[ty * 4 + i][kk], bu, acc_up[i]);
+      }
+    }
+    __syncthreads();
+  }
+  const int n = n0 + tx;
+  if (n >= a.N) return;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int r = ty * 4 + i;
+    if (r < count) gg_store(a, g, orow[r], n, acc[i], acc_up[i]);
+  }
+}
+
+#if AXON_BF16
+typedef __attribute__((ext_vector_type(8))) __bf16 gg_bf16x8;
+typedef __attribute__((ext_vector_type(4))) float gg_f32x4;
+
+__device__ inline gg_bf16x8 gg_frag(uint4 v) { return __builtin_bit_cast(gg_bf16x8, v); }
+
+__device__ inline uint4 gg_x_frag(const GroupedArgs& a, long at, bool ok) {
+  if (!ok) return make_uint4(0, 0, 0, 0);
+  if (!a.x_is_f32) return *reinterpret_cast<const uint4*>((const bf16_t*)a.x + at);
+  const float4 lo = *reinterpret_cast<const float4*>((const float*)a.x + at);
+  const float4 hi = *reinterpret_cast<const float4*>((const float*)a.x + at + 4);
+  return make_uint4(pack2_bf16(lo.x, lo.y), pack2_bf16(lo.z, lo.w), pack2_bf16(hi.x, hi.y), pack2_bf16(hi.z, hi.w));
+}
+
+// 16 rows x 64 columns a block of four waves, a wave 16 columns: W rows as the MFMA's first
+// operand, X rows as its second, both straight from memory (lane l holds row l % 16, the eight k
+// from 8 (l / 16)); lane l ends with row l % 16 of the columns 4 (l / 16) .. + 3.  Four steps of
+// 32 k are asked for before the first is multiplied.
+template <bool GLU>
+__global__ void __launch_bounds__(256) grouped_gemm_mfma_kernel(GroupedArgs a) {
+  int g, first, count;
+  if (!gg_tile(a, g, first, count)) return;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int n0 = blockIdx.y * GG_COLS + wave * 16;
+  if (n0 >= a.N) return;
+  const int r = lane & 15, kq = (lane >> 4) * 8;
+  const bool row_ok = r < count;
+  const int rr = first + min(r, count - 1);
+  const int xr = a.x_rows ? a.x_rows[rr] : rr;
+  const int orow = a.out_rows ? a.out_rows[rr] : rr;
+  const long x_at = (long)xr * a.x_row_stride + (long)g * a.x_group_stride + kq;
+  const int w_rows = GLU ? 2 * a.N : a.N;
+  const bool col_ok = n0 + r < a.N;
+  const bf16_t* wrow = a.w + ((long)g * w_rows + min(n0 + r, a.N - 1)) * a.K + kq;
+  const bf16_t* urow = wrow + (long)a.N * a.K;
+  gg_f32x4 acc = {0.0f, 0.0f, 0.0f, 0.0f}, acc_up = {0.0f, 0.0f, 0.0f, 0.0f};
+  const uint4 zero = make_uint4(0, 0, 0, 0);
+  int k0 = 0;
+  for (; k0 + 128 <= a.K; k0 += 128) {
+    uint4 xf[4], wf[4], uf[4];
+#pragma unroll
+    for (int s = 0; s < 4; ++s) {
+      xf[s] = gg_x_frag(a, x_at + k0 + 32 * s, row_ok);
+      wf[s] = col_ok ? *reinterpret_cast<const uint4*>(wrow + k0 + 32 * s) : zero;
+      if (GLU) uf[s] = col_ok ? *reinterpret_cast<const uint4*>(urow + k0 + 32 * s) : zero;
+    }
+#pragma unroll
+    for (int s = 0; s < 4; ++s) {
+      acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(gg_frag(wf[s]), gg_frag(xf[s]), acc, 0, 0, 0);
+      if (GLU) acc_up = __builtin_amdgcn_mfma_f32_16x16x32_bf16(gg_frag(uf[s]), gg_frag(xf[s]), acc_up, 0, 0, 0);
+    }
+  }
+  for (; k0 < a.K; k0 += 32) {
+    const uint4 xf = gg_x_frag(a, x_at + k0, row_ok);
+    const uint4 wf = col_ok ? *reinterpret_cast<const uint4*>(wrow + k0) : zero;
+    acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(gg_frag(wf), gg_frag(xf), acc, 0, 0, 0);
+    if (GLU) {
+      const uint4 uf = col_ok ? *reinterpret_cast<const uint4*>(urow + k0) : zero;
+      acc_up = __builtin_amdgcn_mfma_f32_16x16x32_bf16(gg_frag(uf), gg_frag(xf), acc_up, 0, 0, 0);
+    }
+  }
+  if (!row_ok) return;
+#pragma unroll
+  for (int c = 0; c < 4; ++c) {
+    const int n = n0 + (lane >> 4) * 4 + c;
+    if (n < a.N) gg_store(a, g, orow, n, acc[c], acc_up[c]);
+  }
+}
+#endif
+
+}  // namespace
+
+extern "C" int axk_grouped_gemm_uses_mfma(int k, int x_is_f32, long x_row_stride, long x_group_stride) {
+#if AXON_BF16
+  const int per16 = x_is_f32 ? 4 : 8;     // elements of X in 16 bytes
+  return k % 32 == 0 && x_row_stride % per16 == 0 && x_group_stride % per16 == 0;
+#else
+  return 0;
+#endif
+}
+
+extern "C" int axk_grouped_gemm(const void* x, int x_is_f32, long x_row_stride, long x_group_stride, const int32_t* x_rows,
+                                const void* w, const void* bias, int bias_is_f32, void* out, int out_is_f32,
+                                long out_row_stride, long out_group_stride, const int32_t* out_rows, const float* gate,
+                                long gate_row_stride, int glu, float glu_limit, float glu_alpha, const int32_t* tiles,
+                                const int32_t* n_tiles, int max_tiles, int m, int n, int k, int groups, void* stream) {
+  AXK_REQUIRE(m >= 0 && n > 0 && k > 0 && groups > 0, "grouped_gemm: bad sizes M=%d N=%d K=%d groups=%d", m, n, k, groups);
+  AXK_REQUIRE((tiles == nullptr) == (n_tiles == nullptr) && (tiles == nullptr || max_tiles >= 0),
+              "grouped_gemm: a list of tiles comes with its length and the most tiles there can be");
+  AXK_REQUIRE(tiles != nullptr || (x_rows == nullptr && out_rows == nullptr),
+              "grouped_gemm: rows are named only beside a list of tiles");
+  const int row_tiles = tiles ? max_tiles : ceil_div(m, GG_ROWS);
+  if (row_tiles == 0) return 0;
+  AXK_REQUIRE(groups <= 65535 && ceil_div(n, GG_COLS) <= 65535, "grouped_gemm: %d groups of %d columns are too many", groups, n);
+  GroupedArgs a{x, x_is_f32, x_row_stride, x_group_stride, x_rows, (const elem_t*)w, bias, bias_is_f32, out, out_is_f32,
+                out_row_stride, out_group_stride, out_rows, gate, gate_row_stride, glu, glu_limit, glu_alpha, tiles, n_tiles,
+                m, n, k, groups};
+  dim3 grid(row_tiles, ceil_div(n, GG_COLS), tiles ? 1 : groups);
+  hipStream_t s = (hipStream_t)stream;
+#if AXON_BF16
+  if (axk_grouped_gemm_uses_mfma(k, x_is_f32, x_row_stride, x_group_stride) && ((uintptr_t)x & 15) == 0 &&
+      ((uintptr_t)w & 15) == 0) {
+    if (glu) { AXK_INSTANCE(INST_GROUPED_GEMM, 1, 1); grouped_gemm_mfma_kernel<true><<<grid, 256, 0, s>>>(a); }
+    else { AXK_INSTANCE(INST_GROUPED_GEMM, 1, 0); grouped_gemm_mfma_kernel<false><<<grid, 256, 0, s>>>(a); }
+    AXK_LAUNCH_CHECK("grouped_gemm");
+    return 0;
+  }
+#endif
+  if (glu) { AXK_INSTANCE(INST_GROUPED_GEMM, 0, 1); grouped_gemm_fma_kernel<true><<<grid, 256, 0, s>>>(a); }
+  else { AXK_INSTANCE(INST_GROUPED_GEMM, 0, 0); grouped_gemm_fma_kernel<false><<<grid, 256, 0, s>>>(a); }
+  AXK_LAUNCH_CHECK("grouped_gemm");
+  return 0;
+}

@@ -15,7 +15,7 @@ namespace {
 
 const char* const KIND_NAMES[INST_KINDS] = {"gemm_fma", "gemm_tile", "gemm_stream", "gemm_normed", "gemm_rows",
                                             "gemm_split_reduce", "attention_rows", "attention_prefill",
-                                            "attention_decode", "rmsnorm"};
+                                            "attention_decode", "rmsnorm", "grouped_gemm"};
 
 struct Registry {
   std::mutex lock;

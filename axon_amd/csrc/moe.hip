@@ -1,0 +1,117 @@
+// Routing for a mixture of experts: the `top` largest of a token's router logits, their softmax,
+// and the (token, chosen expert) pairs listed expert by expert in tiles of up to 16 rows, which
+// the grouped product takes as its work list.  Everything stays on the device: the launches of a
+// step depend on the number of tokens alone.
+#include "api.h"
+#include "common.h"
+
+namespace {
+
+// One thread per token.  The largest logit first; of equal logits the lower expert.  Weights:
+// exp(z - z_first) over the sum of these, added in the order chosen.
+__global__ void route_topk_kernel(const float* __restrict__ logits, int n_tokens, int n_experts, int top,
+                                  int32_t* __restrict__ experts, float* __restrict__ weights) {
+  const int t = blockIdx.x * blockDim.x + threadIdx.x;
+  if (t >= n_tokens) return;
+  const float* z = logits + (long)t * n_experts;
+  int32_t* chosen = experts + (long)t * top;
+  float* w = weights + (long)t * top;
+  float first = 0.0f, sum = 0.0f;
+  for (int k = 0; k < top; ++k) {
+    int best = -1;
+    float best_z = 0.0f;
+    for (int e = 0; e < n_experts; ++e) {
+      bool taken = false;
+      for (int j = 0; j < k; ++j) taken |= chosen[j] == e;
+      if (taken) continue;
+      const float v = z[e];
+      if (best < 0 || v > best_z) { best = e; best_z = v; }
+    }
+    chosen[k] = best;
+    if (k == 0) first = best_z;
+    const float p = expf(best_z - first);
+    w[k] = p;
+    sum += p;
+  }
+  for (int k = 0; k < top; ++k) w[k] = w[k] / sum;
+}
+
+// One block.  pairs p = t top + k in expert order -> sorted [n_pairs], with the token of each
+// (sorted_tokens); tiles [.][3] = (expert, first place in sorted, count <= 16), *n_tiles of them.
+// Which place a pair gets inside its expert's stretch is not fixed (atomic counters); no result
+// depends on it: every row of a product is a chain of its own.
+__global__ void __launch_bounds__(1024)
+route_sort_kernel(const int32_t* __restrict__ experts, int n_pairs, int n_experts, int top, int32_t* __restrict__ sorted,
+                  int32_t* __restrict__ sorted_tokens, int32_t* __restrict__ tiles, int32_t* __restrict__ n_tiles) {
+  extern __shared__ int counts[];              // [n_experts] counts, then [n_experts] next free places
+  int* next = counts + n_experts;
+  for (int e = threadIdx.x; e < n_experts; e += blockDim.x) counts[e] = 0;
+  __syncthreads();
+  for (int p = threadIdx.x; p < n_pairs; p += blockDim.x) atomicAdd(&counts[experts[p]], 1);
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int at = 0, tile = 0;
+    for (int e = 0; e < n_experts; ++e) {
+      const int n = counts[e];
+      next[e] = at;
+      for (int i = 0; i < n; i += 16) {
+        tiles[3 * tile] = e; tiles[3 * tile + 1] = at + i; tiles[3 * tile + 2] = min(16, n - i);
+        ++tile;
+      }
+      at += n;
+    }
+    *n_tiles = tile;
+  }
+  __syncthreads();
+  for (int p = threadIdx.x; p < n_pairs; p += blockDim.x) {
+    const int place = atomicAdd(&next[experts[p]], 1);
+    sorted[place] = p;
+    sorted_tokens[place] = p / top;
+  }
+}
+
+// y[t, :] (+)= sum_k weights[t, k] rows[t top + k, :], k ascending.
+__global__ void route_combine_kernel(const float* __restrict__ rows, const float* __restrict__ weights, float* __restrict__ y,
+                                     int top, int width, int accumulate) {
+  const int t = blockIdx.y;
+  const int c = blockIdx.x * blockDim.x + threadIdx.x;
+  if (c >= width) return;
+  float acc = accumulate ? y[(long)t * width + c] : 0.0f;
+  for (int k = 0; k < top; ++k) acc = fmaf(weights[(long)t * top + k], rows[((long)t * top + k) * width + c], acc);
+  y[(long)t * width + c] = acc;
+}
+
+}  // namespace
+
+extern "C" int axk_route_topk(const float* logits, int n_tokens, int n_experts, int top, int32_t* experts, float* weights,
+                              void* stream) {
+  AXK_REQUIRE(n_tokens >= 0 && n_experts > 0 && top > 0 && top <= n_experts, "route_topk: %d tokens, %d of %d experts",
+              n_tokens, top, n_experts);
+  if (n_tokens == 0) return 0;
+  route_topk_kernel<<<ceil_div(n_tokens, 64), 64, 0, (hipStream_t)stream>>>(logits, n_tokens, n_experts, top, experts, weights);
+  AXK_LAUNCH_CHECK("route_topk");
+  return 0;
+}
+
+extern "C" int axk_route_max_tiles(int n_pairs, int n_experts) { return ceil_div(n_pairs, 16) + n_experts; }
+
+extern "C" int axk_route_sort(const int32_t* experts, int n_pairs, int n_experts, int top, int32_t* sorted,
+                              int32_t* sorted_tokens, int32_t* tiles, int32_t* n_tiles, void* stream) {
+  AXK_REQUIRE(n_pairs >= 0 && n_experts > 0 && top > 0 && n_experts <= 4096, "route_sort: %d pairs, %d experts", n_pairs,
+              n_experts);
+  route_sort_kernel<<<1, 1024, 2 * n_experts * sizeof(int), (hipStream_t)stream>>>(experts, n_pairs, n_experts, top, sorted,
+                                                                                  sorted_tokens, tiles, n_tiles);
+  AXK_LAUNCH_CHECK("route_sort");
+  return 0;
+}
+
+extern "C" int axk_route_combine(const float* rows, const float* weights, float* y, int n_tokens, int top, int width,
+                                 int accumulate, void* stream) {
+  AXK_REQUIRE(n_tokens >= 0 && top > 0 && width > 0 && n_tokens <= 65535, "route_combine: T=%d top=%d width=%d", n_tokens, top,
+              width);
+  if (n_tokens == 0) return 0;
+  dim3 grid(ceil_div(width, 256), n_tokens);
+  route_combine_kernel<<<grid, 256, 0, (hipStream_t)stream>>>(rows, weights, y, top, width, accumulate);
+  AXK_LAUNCH_CHECK("route_combine");
+  return 0;
+}

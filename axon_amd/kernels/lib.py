@@ -8,7 +8,7 @@ other implementation behind these calls: without the library they fail.
 from __future__ import annotations
 
 import ctypes
-from ctypes import c_char_p, c_float, c_int, c_void_p
+from ctypes import c_char_p, c_float, c_int, c_long, c_void_p
 from typing import Dict, List, Optional, Sequence
 
 import numpy as np
@@ -73,6 +73,28 @@ _SIGNATURES = {
     "axk_topk": [c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
                  c_void_p, c_void_p],
     "axk_topk_workspace": [c_int, c_int, c_int],
+    "axk_embed_scaled": [c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_float, c_void_p],
+    "axk_norm_add": [c_void_p, c_void_p, c_int, c_float, c_float, c_void_p, c_void_p, c_int, c_int, c_void_p],
+    "axk_round_rows": [c_void_p, c_void_p, c_long, c_void_p],
+    "axk_activation": [c_void_p, c_long, c_int, c_void_p],
+    "axk_clamped_glu": [c_void_p, c_void_p, c_int, c_int, c_float, c_float, c_void_p],
+    "axk_grouped_gemm_uses_mfma": [c_int, c_int, c_long, c_long],
+    "axk_grouped_gemm": [c_void_p, c_int, c_long, c_long, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_long, c_long,
+                         c_void_p, c_void_p, c_long, c_int, c_float, c_float, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
+                         c_int, c_void_p],
+    "axk_route_topk": [c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p],
+    "axk_route_max_tiles": [c_int, c_int],
+    "axk_route_sort": [c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p],
+    "axk_route_combine": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
+    "axk_causal_conv": [c_void_p, c_long, c_void_p, c_void_p, c_int, c_void_p, c_long, c_int, c_void_p, c_void_p, c_int, c_int,
+                        c_int, c_void_p],
+    "axk_gated_scan": [c_void_p, c_void_p, c_void_p, c_long, c_void_p, c_long, c_void_p, c_int, c_float, c_void_p, c_long,
+                       c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],
+    "axk_latent_prepare": [c_void_p, c_long, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_int, c_void_p, c_int, c_float,
+                           c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_int, c_void_p],
+    "axk_latent_query_rope": [c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],
+    "axk_latent_attention": [c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
+                             c_int, c_int, c_float, c_void_p],
     "axk_fill_i32": [c_void_p, c_int, c_int, c_void_p],
     "axk_fill_f32": [c_void_p, c_float, c_int, c_void_p],
 }
@@ -181,7 +203,9 @@ class Kernels:
     # what launches kernels: wrapped while a step is profiled
     _LAUNCHING = ("embed", "rmsnorm", "rope_table", "rope_kv_write", "gemm_qkv_rope", "attention", "attention_prefill",
                   "attention_decode", "gemm", "gemm_normed_glu", "gemm_normed_qkv_rope", "swiglu", "argmax", "topk",
-                  "fill_i32", "fill_f32", "call")
+                  "fill_i32", "fill_f32", "call", "norm_add", "round_rows", "activation", "clamped_glu", "grouped_gemm",
+                  "route_topk", "route_sort", "route_combine", "causal_conv", "gated_scan", "latent_prepare",
+                  "latent_query_rope", "latent_attention")
     _MATRIX_AT = {"gemm": 1, "gemm_qkv_rope": 1, "gemm_normed_glu": 3, "gemm_normed_qkv_rope": 3}   # which argument is W
 
     def set_launch_hook(self, hook) -> None:
@@ -241,15 +265,15 @@ class Kernels:
             raise KernelError(f"value cache {tuple(v_cache.shape)} is not [pages, {n_kv_heads}, {head_dim}, {page_size}]")
 
     # ------------------------------------------------------------------ ops
-    def embed(self, tokens: torch.Tensor, table: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    def embed(self, tokens: torch.Tensor, table: torch.Tensor, out: torch.Tensor, scale: float = 1.0) -> torch.Tensor:
         packed = isinstance(table, PackedMatrix)
         self._i32(tokens, "embed tokens"); self._elem(table.data if packed else table, "embed table")
         self._f32(out, "embed out")
         vocab, dim = table.shape
         if out.shape != (tokens.numel(), dim) or not (packed or table.is_contiguous()):
             raise KernelError(f"embed: out {tuple(out.shape)} does not fit {tokens.numel()} tokens of width {dim}")
-        self._check(self.lib.axk_embed(_ptr(tokens), _ptr(table), 1 if packed else 0, _ptr(out), tokens.numel(), dim,
-                                       vocab, _stream()))
+        self._check(self.lib.axk_embed_scaled(_ptr(tokens), _ptr(table), 1 if packed else 0, _ptr(out), tokens.numel(), dim,
+                                              vocab, float(scale), _stream()))
         return out
 
     def rmsnorm(self, x: torch.Tensor, gain: torch.Tensor, eps: float, out: torch.Tensor,
@@ -616,6 +640,201 @@ class Kernels:
                                       _ptr(penalty), _ptr(k_of_row), _ptr(cands), cands.shape[1], rows, n, _ptr(work),
                                       _stream()))
         return cands
+
+    # ------------------------------------------------------------------ a norm on a sublayer's output, roundings, activations
+    def norm_add(self, y: torch.Tensor, gain: torch.Tensor, eps: float, mult: float, x: torch.Tensor,
+                 rounded: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """x += mult * rmsnorm(y, gain, eps), row by row; `rounded` also gets the new x in the compute dtype."""
+        self._f32(y, "norm_add y"); self._f32(x, "norm_add x")
+        if y.shape != x.shape or y.dim() != 2 or gain.numel() != x.shape[1]:
+            raise KernelError(f"norm_add: y {tuple(y.shape)}, x {tuple(x.shape)}, a gain of {gain.numel()}")
+        if rounded is not None:
+            self._elem(rounded, "norm_add rounded")
+            if rounded.shape != x.shape or not rounded.is_contiguous():
+                raise KernelError(f"norm_add: rounded {tuple(rounded.shape)} is not {tuple(x.shape)} contiguous")
+        self._check(self.lib.axk_norm_add(_ptr(y), _ptr(gain), self._vec_flag(gain, "norm_add gain"), float(eps), float(mult),
+                                          _ptr(x), _ptr(rounded), x.shape[0], x.shape[1], _stream()))
+        return x
+
+    def round_rows(self, x: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+        self._f32(x, "round_rows x"); self._elem(out, "round_rows out")
+        if out.numel() != x.numel() or not out.is_contiguous():
+            raise KernelError(f"round_rows: {tuple(x.shape)} into {tuple(out.shape)}")
+        self._check(self.lib.axk_round_rows(_ptr(x), _ptr(out), x.numel(), _stream()))
+        return out
+
+    def activation(self, v: torch.Tensor, kind: str = "gelu_tanh") -> torch.Tensor:
+        self._elem(v, "activation")
+        if kind != "gelu_tanh" or not v.is_contiguous():
+            raise KernelError(f"activation: '{kind}' on a tensor of strides {v.stride()}")
+        self._check(self.lib.axk_activation(_ptr(v), v.numel(), 0, _stream()))
+        return v
+
+    def clamped_glu(self, gate_up: torch.Tensor, out: torch.Tensor, limit: float, alpha: float) -> torch.Tensor:
+        self._elem(gate_up, "clamped_glu in"); self._elem(out, "clamped_glu out")
+        T, F = out.shape
+        if gate_up.shape != (T, 2 * F) or not gate_up.is_contiguous() or not out.is_contiguous():
+            raise KernelError(f"clamped_glu: in {tuple(gate_up.shape)} out {tuple(out.shape)}")
+        self._check(self.lib.axk_clamped_glu(_ptr(gate_up), _ptr(out), T, F, float(limit), float(alpha), _stream()))
+        return out
+
+    # ------------------------------------------------------------------ grouped products
+    def grouped_gemm(self, x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, *, x_group_stride: int, out_group_stride: int,
+                     bias: Optional[torch.Tensor] = None, gate: Optional[torch.Tensor] = None, glu=None, routed=None,
+                     rows: Optional[int] = None) -> torch.Tensor:
+        """out[orow(r), g ogs + n] = epilogue(sum_k x[xrow(r), g xgs + k] w[g, n, k] + bias[g, n]).
+
+        x [rows, >= g xgs + K] float32 or compute dtype, rows may be strided; w [G, N, K] (with `glu`
+        = (limit, alpha): [G, 2 N, K], gate rows then up rows) in the compute dtype; out float32 or
+        compute dtype.  Block-diagonal: every row meets every group.  `routed` = (tiles, n_tiles,
+        max_tiles, x_rows, out_rows), int32 on the device: the listed rows (`rows` of them at
+        most) meet the group their tile names.  `gate` (float32, out's shape): out is multiplied
+        by its sigmoid."""
+        G, NW, K = w.shape
+        N = NW // 2 if glu else NW
+        self._elem(w, "grouped w")
+        if not w.is_contiguous() or x.stride(-1) != 1 or out.stride(-1) != 1 or x.dim() != 2 or out.dim() != 2:
+            raise KernelError("grouped_gemm: w must be contiguous, x and out row-major matrices")
+        for t, what in ((x, "x"), (out, "out")):
+            if t.dtype not in (torch.float32, self.dtype) or not t.is_cuda:
+                raise KernelError(f"grouped_gemm: {what} is {t.dtype} on {t.device}")
+        M = x.shape[0] if rows is None else int(rows)
+        if x.shape[1] < (G - 1) * x_group_stride + K and routed is None or out.shape[1] < (G - 1) * out_group_stride + N and routed is None:
+            raise KernelError(f"grouped_gemm: x {tuple(x.shape)} / out {tuple(out.shape)} do not hold {G} groups of {K} -> {N}")
+        if routed is None and out.shape[0] != M:
+            raise KernelError(f"grouped_gemm: {M} rows in, {out.shape[0]} out")
+        if bias is not None and bias.numel() != G * NW:
+            raise KernelError(f"grouped_gemm: a bias of {bias.numel()} for {G} x {NW}")
+        if gate is not None:
+            if gate.dtype != torch.float32 or not gate.is_cuda or gate.dim() != 2 or gate.shape[0] != out.shape[0] or gate.stride(-1) != 1:
+                raise KernelError(f"grouped_gemm: gate {tuple(gate.shape)} for out {tuple(out.shape)}")
+        tiles = n_tiles = x_rows = out_rows = None
+        max_tiles = 0
+        if routed is not None:
+            tiles, n_tiles, max_tiles, x_rows, out_rows = routed
+            for t in (tiles, n_tiles, x_rows, out_rows):
+                if t is not None:
+                    self._i32(t, "grouped_gemm routing")
+            if x.shape[1] < K or out.shape[1] < N:
+                raise KernelError(f"grouped_gemm: x {tuple(x.shape)} / out {tuple(out.shape)} for {K} -> {N}")
+        limit, alpha = glu if glu else (0.0, 0.0)
+        self._check(self.lib.axk_grouped_gemm(
+            _ptr(x), 1 if x.dtype == torch.float32 else 0, x.stride(0), x_group_stride, _ptr(x_rows), _ptr(w), _ptr(bias),
+            self._vec_flag(bias, "grouped bias"), _ptr(out), 1 if out.dtype == torch.float32 else 0, out.stride(0),
+            out_group_stride, _ptr(out_rows), _ptr(gate), 0 if gate is None else gate.stride(0), 1 if glu else 0, float(limit),
+            float(alpha), _ptr(tiles), _ptr(n_tiles), int(max_tiles), M, N, K, G, _stream()))
+        return out
+
+    # ------------------------------------------------------------------ routing
+    def route_topk(self, logits: torch.Tensor, top: int, experts: torch.Tensor, weights: torch.Tensor) -> None:
+        self._f32(logits, "router logits"); self._i32(experts, "chosen experts"); self._f32(weights, "router weights")
+        T, E = logits.shape
+        if experts.shape != (T, top) or weights.shape != (T, top):
+            raise KernelError(f"route_topk: {tuple(experts.shape)} / {tuple(weights.shape)} for {T} x {top}")
+        self._check(self.lib.axk_route_topk(_ptr(logits), T, E, top, _ptr(experts), _ptr(weights), _stream()))
+
+    def route_max_tiles(self, n_pairs: int, n_experts: int) -> int:
+        return int(self.lib.axk_route_max_tiles(n_pairs, n_experts))
+
+    def route_sort(self, experts: torch.Tensor, n_experts: int, sorted_pairs, sorted_tokens, tiles, n_tiles) -> None:
+        for t in (experts, sorted_pairs, sorted_tokens, tiles, n_tiles):
+            self._i32(t, "route_sort")
+        P = experts.numel()
+        if sorted_pairs.numel() < P or sorted_tokens.numel() < P or tiles.numel() < 3 * self.route_max_tiles(P, n_experts):
+            raise KernelError(f"route_sort: lists too short for {P} pairs of {n_experts} experts")
+        self._check(self.lib.axk_route_sort(_ptr(experts), P, n_experts, experts.shape[-1], _ptr(sorted_pairs), _ptr(sorted_tokens),
+                                            _ptr(tiles), _ptr(n_tiles), _stream()))
+
+    def route_combine(self, rows: torch.Tensor, weights: torch.Tensor, y: torch.Tensor, accumulate: bool = False) -> torch.Tensor:
+        self._f32(rows, "expert rows"); self._f32(weights, "router weights"); self._f32(y, "combine y")
+        T, top = weights.shape
+        if rows.shape != (T * top, y.shape[1]) or y.shape[0] != T:
+            raise KernelError(f"route_combine: rows {tuple(rows.shape)}, weights {tuple(weights.shape)}, y {tuple(y.shape)}")
+        self._check(self.lib.axk_route_combine(_ptr(rows), _ptr(weights), _ptr(y), T, top, y.shape[1], 1 if accumulate else 0,
+                                               _stream()))
+        return y
+
+    # ------------------------------------------------------------------ convolution and recurrence with per-request state
+    def causal_conv(self, x: torch.Tensor, w: torch.Tensor, bias, state: torch.Tensor, state_offset: int, seq_rows: torch.Tensor,
+                    u: torch.Tensor) -> torch.Tensor:
+        """u[t, c] = bias[c] + sum_k w[c, k] x(t - (taps - 1 - k)); x [T, C] in the compute dtype (rows may
+        be strided), inputs before the step from the float32 state rows [slots, >= offset + (taps - 1) C]."""
+        self._elem(x, "conv x"); self._elem(w, "conv w"); self._f32(state, "conv state"); self._f32(u, "conv u")
+        self._i32(seq_rows, "seq_rows")
+        T, C = u.shape
+        if x.shape != (T, C) or x.stride(1) != 1 or w.dim() != 2 or w.shape[0] != C or not w.is_contiguous() or seq_rows.numel() != T:
+            raise KernelError(f"causal_conv: x {tuple(x.shape)}, w {tuple(w.shape)}, u {tuple(u.shape)}")
+        if bias is not None and bias.numel() != C:
+            raise KernelError(f"causal_conv: a bias of {bias.numel()} for {C} channels")
+        self._check(self.lib.axk_causal_conv(_ptr(x), x.stride(0), _ptr(w), _ptr(bias), self._vec_flag(bias, "conv bias"),
+                                             _ptr(state), state.stride(0), int(state_offset), _ptr(seq_rows), _ptr(u), T, C,
+                                             w.shape[1], _stream()))
+        return u
+
+    def gated_scan(self, gates, u, y, x, lam, decay: float, state, spans, seq_rows, out, block_width: int, taps: int):
+        """The gated linear recurrence over each request's tokens (see csrc/recurrent.hip): gates
+        [T, C / block_width, 2 block_width] and u [T, C] float32; y, x [T, C] compute dtype (rows may be
+        strided); state float32 [slots, >= taps C]; spans int32 [n, 3] = (slot, first token, tokens) or
+        None (each token a request of its own in slot seq_rows[t]); out [T, C] compute dtype."""
+        self._f32(gates, "scan gates"); self._f32(u, "scan u"); self._elem(y, "scan y"); self._elem(x, "scan x")
+        self._f32(state, "scan state"); self._elem(out, "scan out"); self._i32(seq_rows, "seq_rows")
+        T, C = u.shape
+        if (gates.shape != (T, 2 * C) and gates.numel() != T * 2 * C) or y.shape != (T, C) or x.shape != (T, C) or out.shape != (T, C) \
+                or y.stride(1) != 1 or x.stride(1) != 1 or not out.is_contiguous() or lam.numel() != C or seq_rows.numel() != T:
+            raise KernelError(f"gated_scan: gates {tuple(gates.shape)}, u {tuple(u.shape)}, y {tuple(y.shape)}, out {tuple(out.shape)}")
+        if spans is not None:
+            self._i32(spans, "scan spans")
+            n = spans.shape[0]
+        else:
+            n = T
+        self._check(self.lib.axk_gated_scan(_ptr(gates), _ptr(u), _ptr(y), y.stride(0), _ptr(x), x.stride(0), _ptr(lam),
+                                            self._vec_flag(lam, "scan lam"), float(decay), _ptr(state), state.stride(0),
+                                            _ptr(spans), n, _ptr(seq_rows), _ptr(out), C, int(block_width), int(taps), _stream()))
+        return out
+
+    # ------------------------------------------------------------------ attention over a latent cache
+    def latent_prepare(self, fused, q_at, q_rank, kv_at, rank, rot, rot_dims, q_gain, kv_gain, eps, table, positions, seq_rows,
+                       block_table, cache, page_size, cq, write_kv=True) -> None:
+        self._f32(fused, "latent fused"); self._f32(table, "rope table"); self._i32(positions, "positions")
+        self._i32(seq_rows, "seq_rows"); self._i32(block_table, "block_table"); self._elem(cache, "latent cache")
+        T = positions.numel()
+        if fused.shape[0] != T or (rot_dims and table.shape != (T, rot_dims // 2, 2)) or seq_rows.numel() != T:
+            raise KernelError(f"latent_prepare: fused {tuple(fused.shape)}, table {tuple(table.shape)} for {T} tokens")
+        if cache.dim() != 4 or tuple(cache.shape[1:]) != (1, page_size, rank + rot) or not cache.is_contiguous():
+            raise KernelError(f"latent_prepare: cache {tuple(cache.shape)} is not [pages, 1, {page_size}, {rank + rot}]")
+        if q_rank:
+            self._elem(cq, "latent cq")
+            if cq.shape != (T, q_rank) or not cq.is_contiguous() or q_gain.numel() != q_rank:
+                raise KernelError(f"latent_prepare: cq {tuple(cq.shape)} for a query latent of {q_rank}")
+        if kv_gain.numel() != rank:
+            raise KernelError(f"latent_prepare: a gain of {kv_gain.numel()} for a latent of {rank}")
+        self._check(self.lib.axk_latent_prepare(
+            _ptr(fused), fused.stride(0), q_at, q_rank, kv_at, rank, rot, rot_dims, _ptr(q_gain), self._vec_flag(q_gain, "q gain"),
+            _ptr(kv_gain), self._vec_flag(kv_gain, "kv gain"), float(eps), _ptr(table), _ptr(positions), _ptr(seq_rows),
+            _ptr(block_table), block_table.shape[-1], _ptr(cache), page_size, _ptr(cq if q_rank else None), T,
+            1 if write_kv else 0, _stream()))
+
+    def latent_query_rope(self, q, dim, rot, rot_dims, table, q_full, rank, heads) -> None:
+        self._f32(q, "latent q"); self._f32(q_full, "latent q_full"); self._f32(table, "rope table")
+        T = q.shape[0]
+        if q.shape != (T, heads * (dim + rot)) or q_full.shape != (T, heads * (rank + rot)):
+            raise KernelError(f"latent_query_rope: q {tuple(q.shape)}, q_full {tuple(q_full.shape)}")
+        self._check(self.lib.axk_latent_query_rope(_ptr(q), dim, rot, rot_dims, _ptr(table), _ptr(q_full), rank, heads, T,
+                                                   _stream()))
+
+    def latent_attention(self, q_full, cache, block_table, positions, seq_rows, o_lat, heads, rank, rot, page_size, window,
+                         scale) -> torch.Tensor:
+        self._f32(q_full, "latent q_full"); self._f32(o_lat, "latent o_lat"); self._elem(cache, "latent cache")
+        self._i32(positions, "positions"); self._i32(seq_rows, "seq_rows"); self._i32(block_table, "block_table")
+        T = positions.numel()
+        if q_full.shape != (T, heads * (rank + rot)) or o_lat.shape != (T, heads * rank) or seq_rows.numel() != T:
+            raise KernelError(f"latent_attention: q_full {tuple(q_full.shape)}, o_lat {tuple(o_lat.shape)} for {T} tokens")
+        if cache.dim() != 4 or tuple(cache.shape[1:]) != (1, page_size, rank + rot) or not cache.is_contiguous():
+            raise KernelError(f"latent_attention: cache {tuple(cache.shape)} is not [pages, 1, {page_size}, {rank + rot}]")
+        self._check(self.lib.axk_latent_attention(_ptr(q_full), _ptr(cache), _ptr(block_table), block_table.shape[-1],
+                                                  _ptr(positions), _ptr(seq_rows), _ptr(o_lat), T, heads, rank, rot, page_size,
+                                                  int(window), float(scale), _stream()))
+        return o_lat
 
     def fill_i32(self, dst: torch.Tensor, value: int) -> None:
         self._i32(dst, "fill")

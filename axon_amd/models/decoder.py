@@ -35,7 +35,8 @@ class DecoderModel:
         self.blocks = []
         for layer in spec.layers:
             mixer = build_part("mixer", layer.mixer, layer.prefix)
-            ffn = build_part("feed_forward", layer.feed_forward, layer.prefix)
+            # a layer may have no feed-forward (its block then has to be one that takes none)
+            ffn = build_part("feed_forward", layer.feed_forward, layer.prefix) if layer.feed_forward is not None else None
             self.blocks.append(build_block(layer.block, layer.norm, mixer, ffn, layer.prefix))
         self.final_norm = build_part("norm", spec.final_norm)
         self.head = build_part("head", spec.head)
@@ -134,7 +135,7 @@ class DecoderModel:
     def run_is_graph_safe(self, i: int) -> bool:
         """Whether run i's block and its parts are all fixed launch sequences (see Part.graph_safe)."""
         block = self.blocks[self.order[i].layer]
-        return all(getattr(p, "graph_safe", False) for p in (block, block.mixer, block.feed_forward))
+        return all(getattr(p, "graph_safe", False) for p in (block, block.mixer, block.feed_forward) if p is not None)
 
     def ends_are_graph_safe(self) -> bool:
         """Whether what runs before the first run and behind the last (`embed`, `logits`) is a fixed

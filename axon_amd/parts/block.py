@@ -8,6 +8,9 @@ from __future__ import annotations
 
 from typing import List
 
+import torch
+
+from ..config.base import ConfigError
 from .base import Block, CacheBinding, TensorDecl, register_block
 
 # A norm behind a product whose kernel holds the finished rows anyway can be written by that
@@ -59,4 +62,59 @@ class PreNormBlock(Block):
             self.feed_forward.forward(ctx, h, x)
 
 
+class SublayerNormBlock(Block):
+    """x += mult * norm1(mixer(x)); x += mult * norm2(feed_forward(x)): the norms sit on the sublayers'
+    outputs, the sublayers read the residual stream itself (rounded to the compute dtype for their
+    products), and a layer may have no feed-forward.  The norm, the scaling and the sum are one
+    32-bit pass over the sublayer's 32-bit output, which also leaves the new rows rounded for the
+    next sublayer.  The norms are RMS norms (they hand over a gain and an eps).  `residual_mult`
+    comes with the norm's parameters."""
+    graph_safe = True
+    norm1_name = "norm1"
+    norm2_name = "norm2"
+
+    def __init__(self, norm_factory, mixer, feed_forward, prefix):
+        super().__init__(norm_factory, mixer, feed_forward, prefix)
+        self.norm1 = norm_factory(self.norm1_name)
+        self.norm2 = norm_factory(self.norm2_name) if feed_forward is not None else None
+        for norm in (self.norm1, self.norm2):
+            if norm is not None and not (hasattr(norm, "gain") and hasattr(norm, "eps")):
+                raise ConfigError("a norm on a sublayer's output is an RMS norm (a gain and an eps)")
+        self.mult = float(self.norm1.params.get("residual_mult", 1.0))
+
+    def parts(self):
+        return [p for p in (self.norm1, self.mixer, self.norm2, self.feed_forward) if p is not None]
+
+    def tensors(self) -> List[TensorDecl]:
+        return [d for p in self.parts() for d in p.tensors()]
+
+    def load(self, store, rt) -> None:
+        for part in self.parts():
+            part.load(store, rt)
+
+    @staticmethod
+    def _run(part, ctx, y, *args) -> None:
+        """y = part(...): stored by the part's last product where it can, else added into zeros."""
+        if getattr(part, "stores_output", False):
+            part.forward(ctx, *args, y, accumulate=False)
+        else:
+            ctx.rt.k.fill_f32(y.view(-1), 0.0)
+            part.forward(ctx, *args, y)
+
+    def forward(self, ctx, binding: CacheBinding, x, normed=None, following=None) -> None:
+        k, rt = ctx.rt.k, ctx.rt
+        exact = rt.dtype == torch.float32            # the 32-bit path: the sublayers read x as it is
+        h = x if exact else k.round_rows(x, ctx.ws.take(tuple(x.shape), rt.dtype))
+        y = ctx.ws.take(tuple(x.shape), torch.float32)
+        self._run(self.mixer, ctx, y, binding, h)
+        if self.feed_forward is None:
+            k.norm_add(y, self.norm1.gain, self.norm1.eps, self.mult, x)
+            return
+        h = x if exact else ctx.ws.take(tuple(x.shape), rt.dtype)
+        k.norm_add(y, self.norm1.gain, self.norm1.eps, self.mult, x, None if exact else h)
+        self._run(self.feed_forward, ctx, y, h)
+        k.norm_add(y, self.norm2.gain, self.norm2.eps, self.mult, x)
+
+
 register_block("prenorm", PreNormBlock)
+register_block("sublayer_norm", SublayerNormBlock)

@@ -22,6 +22,7 @@ class TokenEmbedding(Part):
         self.vocab = int(params["vocab_size"])
         self.hidden = int(params["hidden_size"])
         self.name = prefix + params["tensor"]
+        self.scale = float(params.get("scale", 1.0))      # every row is multiplied by it (32-bit)
         self.table = None            # row-major, or a head's packed matrix (see LMHead.load)
 
     def tensors(self) -> List[TensorDecl]:
@@ -39,7 +40,7 @@ class TokenEmbedding(Part):
     def forward(self, ctx, out=None):
         if out is None:
             out = ctx.ws.take((ctx.n_tokens, self.hidden), torch.float32)
-        return ctx.rt.k.embed(ctx.tokens, self.table, out)
+        return ctx.rt.k.embed(ctx.tokens, self.table, out, self.scale)
 
 
 class LMHead(Part):

@@ -1,0 +1,107 @@
+"""Attention whose keys and values go through a shared latent (multi-head latent attention).
+
+From the input h: the query latent c_q = rmsnorm(Wdq h), q = Wuq c_q, laid out head by head as
+[dim unrotated, rot_dim rotated]; Wdkv h gives kv_rank rows that, RMS-normed, are the latent c,
+and rot_dim more that are one rotated key part shared by all heads.  A head's unrotated key is
+Wuk c and its value Wuv c; the score is (q_unrot . k_unrot + q_rot . k_rot) * scale over a
+causal window; the concatenated heads are multiplied by sigmoid(Wg h) and projected by Wo.
+
+Only c and the rotated key part are cached (one row of kv_rank + rot_dim per position), and the
+keys and values are never built: the unrotated query is carried into the latent space
+(q_lat = Wuk^T q_unrot, a per-head product), attention runs there, and the head's output is
+Wuv (sum_j p_j c_j), a second per-head product.
+
+Parameters: `hidden_size`, `heads`, `dim`, `rot_dim`, `vdim`, `kv_rank`, `q_rank`, `scale`,
+`window` (0: all earlier positions), `eps` (of the latents' norms), `gated` (the sigmoid gate),
+`position` (a PartSpec of the rotation), `names`.
+"""
+from __future__ import annotations
+
+from typing import List, Optional
+
+import torch
+
+from ..config.base import ConfigError
+from ..kernels import MODE_ADD_F32, MODE_STORE_F32
+from .base import CacheBinding, CacheSpec, Mixer, TensorDecl, build_part, register_mixer
+
+
+class LatentAttention(Mixer):
+    graph_safe = True
+    stores_output = True
+
+    def __init__(self, params, prefix=""):
+        super().__init__(params, prefix)
+        p = params
+        self.hidden, self.heads = int(p["hidden_size"]), int(p["heads"])
+        self.dim, self.rot, self.vdim = int(p["dim"]), int(p["rot_dim"]), int(p["vdim"])
+        self.kv_rank, self.q_rank = int(p["kv_rank"]), int(p["q_rank"])
+        self.scale, self.window, self.eps = float(p["scale"]), int(p.get("window", 0)), float(p["eps"])
+        self.gated = bool(p.get("gated", True))
+        self.position = build_part("position", p["position"]) if p.get("position") is not None and self.rot > 0 else None
+        self.rot_dims = self.position.rotary_dim if self.position is not None else 0
+        if self.rot_dims > self.rot:
+            raise ConfigError(f"{self.rot_dims} rotated dims in a rotated part of {self.rot}")
+        if self.kv_rank > 1024:
+            raise ConfigError(f"a key/value latent of {self.kv_rank} is more than the attention kernel's 1024")
+        names = p.get("names", {})
+        base = prefix + names.get("scope", "mix.")
+        self.n = {k: base + names.get(k, k) for k in ("dq", "uq", "dkv", "uk", "uv", "g", "o")}
+
+    def tensors(self) -> List[TensorDecl]:
+        n, H = self.n, self.heads
+        t = [TensorDecl(n["dq"], (self.q_rank, self.hidden)), TensorDecl(n["dq"] + ".norm", (self.q_rank,), "gain"),
+             TensorDecl(n["uq"], (H * (self.dim + self.rot), self.q_rank)),
+             TensorDecl(n["dkv"], (self.kv_rank + self.rot, self.hidden)), TensorDecl(n["dkv"] + ".norm", (self.kv_rank,), "gain"),
+             TensorDecl(n["uk"], (H * self.dim, self.kv_rank)), TensorDecl(n["uv"], (H * self.vdim, self.kv_rank)),
+             TensorDecl(n["o"], (self.hidden, H * self.vdim))]
+        if self.gated:
+            t.append(TensorDecl(n["g"], (H * self.vdim, self.hidden)))
+        return t
+
+    def cache_spec(self) -> Optional[CacheSpec]:
+        return CacheSpec(entries=1, heads=1, head_dim=self.kv_rank + self.rot, window=self.window)
+
+    def load(self, store, rt) -> None:
+        n, H = self.n, self.heads
+        down = [n["dq"], n["dkv"]] + ([n["g"]] if self.gated else [])
+        self.w_down = rt.k.prepare_weight(store.fused_matrix(down))
+        self.q_gain, self.kv_gain = store.vector(n["dq"] + ".norm"), store.vector(n["dkv"] + ".norm")
+        self.w_uq = rt.k.prepare_weight(store.matrix(n["uq"]))
+        # per head: Wuk^T [kv_rank, dim] carries a query into the latent space, Wuv [vdim, kv_rank] a latent out of it
+        self.w_uk_t = store.matrix(n["uk"]).view(H, self.dim, self.kv_rank).transpose(1, 2).contiguous()
+        self.w_uv = store.matrix(n["uv"]).view(H, self.vdim, self.kv_rank).contiguous()
+        self.w_o = rt.k.prepare_weight(store.matrix(n["o"]))
+        for name in (n["uq"], n["uk"], n["o"]):
+            store.forget(name)
+        if self.position is not None:
+            self.position.load(store, rt)
+
+    def forward(self, ctx, binding: CacheBinding, h, out, accumulate: bool = True) -> None:
+        k, T, H = ctx.rt.k, h.shape[0], self.heads
+        group = ctx.cache.group(binding.group)
+        (cache,) = group.layer(binding.index)
+        n_down = self.q_rank + self.kv_rank + self.rot + (H * self.vdim if self.gated else 0)
+        down = ctx.ws.take((T, n_down), torch.float32)
+        k.gemm(h, self.w_down, down, None, MODE_STORE_F32)
+        table = self.position.tables(ctx) if self.position is not None else ctx.no_rotation()
+        cq = ctx.ws.take((T, self.q_rank), ctx.rt.dtype)
+        k.latent_prepare(down, 0, self.q_rank, self.q_rank, self.kv_rank, self.rot, self.rot_dims, self.q_gain, self.kv_gain,
+                         self.eps, table, ctx.positions, ctx.seq_rows, group.block_table, cache, group.page_size, cq,
+                         binding.writes)
+        q = ctx.ws.take((T, H * (self.dim + self.rot)), torch.float32)
+        k.gemm(cq, self.w_uq, q, None, MODE_STORE_F32)
+        width = self.kv_rank + self.rot
+        q_full = ctx.ws.take((T, H * width), torch.float32)
+        k.latent_query_rope(q, self.dim, self.rot, self.rot_dims, table, q_full, self.kv_rank, H)
+        k.grouped_gemm(q, self.w_uk_t, q_full, x_group_stride=self.dim + self.rot, out_group_stride=width)
+        o_lat = ctx.ws.take((T, H * self.kv_rank), torch.float32)
+        k.latent_attention(q_full, cache, group.block_table, ctx.positions, ctx.seq_rows, o_lat, H, self.kv_rank, self.rot,
+                           group.page_size, self.window, self.scale)
+        att = ctx.ws.take((T, H * self.vdim), ctx.rt.dtype)
+        gate = down[:, self.q_rank + self.kv_rank + self.rot:] if self.gated else None
+        k.grouped_gemm(o_lat, self.w_uv, att, x_group_stride=self.kv_rank, out_group_stride=self.vdim, gate=gate)
+        k.gemm(att, self.w_o, out, None, MODE_ADD_F32 if accumulate else MODE_STORE_F32)
+
+
+register_mixer("latent_attention", LatentAttention)

@@ -9,7 +9,8 @@ from __future__ import annotations
 
 from typing import List
 
-from ..kernels import MODE_ADD_F32, MODE_SWIGLU, PackedMatrix
+from ..config.base import ConfigError
+from ..kernels import MODE_ADD_F32, MODE_STORE, MODE_STORE_F32, MODE_SWIGLU, PackedMatrix
 from .base import FeedForward, PrecedingNorm, TensorDecl, register_feed_forward
 
 
@@ -54,3 +55,72 @@ class SwiGLUMLP(FeedForward):
 
 
 register_feed_forward("swiglu_mlp", SwiGLUMLP)
+
+
+class DenseMLP(FeedForward):
+    """down(act(up h)): a plain two-matrix feed-forward.  Parameters: `hidden_size`, `ff`,
+    `activation` ("gelu_tanh": 0.5 z (1 + tanh(sqrt(2 / pi) (z + 0.044715 z^3)))), `names` (scope "mlp.", up, down)."""
+    graph_safe = True
+    stores_output = True
+
+    def __init__(self, params, prefix=""):
+        super().__init__(params, prefix)
+        self.hidden, self.ff = int(params["hidden_size"]), int(params["ff"])
+        self.activation = params.get("activation", "gelu_tanh")
+        if self.activation != "gelu_tanh":
+            raise ConfigError(f"activation '{self.activation}' is not known (gelu_tanh)")
+        names = params.get("names", {})
+        base = prefix + names.get("scope", "mlp.")
+        self.n = {k: base + names.get(k, k) for k in ("up", "down")}
+
+    def tensors(self) -> List[TensorDecl]:
+        return [TensorDecl(self.n["up"], (self.ff, self.hidden)), TensorDecl(self.n["down"], (self.hidden, self.ff))]
+
+    def load(self, store, rt) -> None:
+        self.w_up = rt.k.prepare_weight(store.matrix(self.n["up"]))
+        self.w_down = rt.k.prepare_weight(store.matrix(self.n["down"]))
+        for name in self.n.values():
+            store.forget(name)
+
+    def forward(self, ctx, h, out, accumulate: bool = True) -> None:
+        k = ctx.rt.k
+        act = ctx.ws.take((h.shape[0], self.ff), ctx.rt.dtype)
+        k.gemm(h, self.w_up, act, None, MODE_STORE)
+        k.activation(act, self.activation)
+        k.gemm(act, self.w_down, out, None, MODE_ADD_F32 if accumulate else MODE_STORE_F32)
+
+
+class ClampedGLUMLP(FeedForward):
+    """down(g sigmoid(alpha g) (u + 1)) with g = min(gate h, limit), u = clamp(up h, -limit, limit); no
+    biases.  Parameters: `hidden_size`, `ff`, `limit`, `alpha` (default 1.702), `names` (scope "mlp.", gate, up, down)."""
+    graph_safe = True
+    stores_output = True
+
+    def __init__(self, params, prefix=""):
+        super().__init__(params, prefix)
+        self.hidden, self.ff = int(params["hidden_size"]), int(params["ff"])
+        self.limit, self.alpha = float(params["limit"]), float(params.get("alpha", 1.702))
+        names = params.get("names", {})
+        base = prefix + names.get("scope", "mlp.")
+        self.n = {k: base + names.get(k, k) for k in ("gate", "up", "down")}
+
+    def tensors(self) -> List[TensorDecl]:
+        return [TensorDecl(self.n["gate"], (self.ff, self.hidden)), TensorDecl(self.n["up"], (self.ff, self.hidden)),
+                TensorDecl(self.n["down"], (self.hidden, self.ff))]
+
+    def load(self, store, rt) -> None:
+        self.w_gate_up = rt.k.prepare_weight(store.fused_matrix([self.n["gate"], self.n["up"]]))
+        self.w_down = rt.k.prepare_weight(store.matrix(self.n["down"]))
+        store.forget(self.n["down"])
+
+    def forward(self, ctx, h, out, accumulate: bool = True) -> None:
+        k, T = ctx.rt.k, h.shape[0]
+        gate_up = ctx.ws.take((T, 2 * self.ff), ctx.rt.dtype)
+        k.gemm(h, self.w_gate_up, gate_up, None, MODE_STORE)
+        act = ctx.ws.take((T, self.ff), ctx.rt.dtype)
+        k.clamped_glu(gate_up, act, self.limit, self.alpha)
+        k.gemm(act, self.w_down, out, None, MODE_ADD_F32 if accumulate else MODE_STORE_F32)
+
+
+register_feed_forward("dense_mlp", DenseMLP)
+register_feed_forward("clamped_glu_mlp", ClampedGLUMLP)

@@ -1,0 +1,95 @@
+"""A mixture of experts: each token goes through the `top` experts its router logits rank first,
+weighted by the softmax over those logits alone; a shared expert, if any, sees every token.
+
+Router logits are 32-bit (Wr h with h in the compute dtype).  An expert is a gated unit with
+clamps: g = min(Wgate h, limit), u = clamp(Wup h, -limit, limit), out = Wdown (g sigmoid(alpha g)
+(u + 1)), without biases.  The (token, chosen expert) pairs are listed expert by expert on the
+device and two grouped products (gate|up with the activation in its epilogue, then down) run
+over the list; a token's rows are then added in the order of its router's ranking.
+
+Parameters: `hidden_size`, `experts`, `top`, `ff`, `limit`, `alpha` (default 1.702), `shared`
+(None, or {"ff", "limit"}), `names` (scope "mlp.", router, expert "e{}.", shared "shared.").
+"""
+from __future__ import annotations
+
+from typing import List
+
+import torch
+
+from ..config.base import ConfigError, PartSpec
+from ..kernels import MODE_STORE_F32
+from .base import FeedForward, TensorDecl, build_part, register_feed_forward
+
+
+class RoutedExperts(FeedForward):
+    graph_safe = True
+    stores_output = True
+
+    def __init__(self, params, prefix=""):
+        super().__init__(params, prefix)
+        p = params
+        self.hidden, self.n_experts, self.top = int(p["hidden_size"]), int(p["experts"]), int(p["top"])
+        self.ff, self.limit, self.alpha = int(p["ff"]), float(p["limit"]), float(p.get("alpha", 1.702))
+        if not 1 <= self.top <= self.n_experts:
+            raise ConfigError(f"{self.top} of {self.n_experts} experts a token")
+        names = p.get("names", {})
+        self.base = prefix + names.get("scope", "mlp.")
+        self.router_name = self.base + names.get("router", "router")
+        self.expert_scope = names.get("expert", "e{}.")
+        self.shared = None
+        if p.get("shared"):
+            sh = p["shared"]
+            self.shared = build_part("feed_forward", PartSpec("clamped_glu_mlp", {
+                "hidden_size": self.hidden, "ff": int(sh["ff"]), "limit": float(sh["limit"]),
+                "alpha": float(sh.get("alpha", self.alpha)),
+                "names": {"scope": names.get("scope", "mlp.") + names.get("shared", "shared.")}}), prefix)
+
+    def _expert(self, e: int, which: str) -> str:
+        return self.base + self.expert_scope.format(e) + which
+
+    def tensors(self) -> List[TensorDecl]:
+        t = [TensorDecl(self.router_name, (self.n_experts, self.hidden))]
+        for e in range(self.n_experts):
+            t += [TensorDecl(self._expert(e, "gate"), (self.ff, self.hidden)), TensorDecl(self._expert(e, "up"), (self.ff, self.hidden)),
+                  TensorDecl(self._expert(e, "down"), (self.hidden, self.ff))]
+        return t + (self.shared.tensors() if self.shared is not None else [])
+
+    def load(self, store, rt) -> None:
+        self.w_router = rt.k.prepare_weight(store.matrix(self.router_name))
+        E = self.n_experts
+        # every expert's gate rows, then its up rows: [experts, 2 ff, hidden]; and [experts, hidden, ff]
+        self.w_gate_up = torch.empty((E, 2 * self.ff, self.hidden), dtype=rt.dtype, device=rt.device)
+        self.w_down = torch.empty((E, self.hidden, self.ff), dtype=rt.dtype, device=rt.device)
+        for e in range(E):
+            self.w_gate_up[e, :self.ff].copy_(store.matrix(self._expert(e, "gate")))
+            self.w_gate_up[e, self.ff:].copy_(store.matrix(self._expert(e, "up")))
+            self.w_down[e].copy_(store.matrix(self._expert(e, "down")))
+            for which in ("gate", "up", "down"):
+                store.forget(self._expert(e, which))
+        if self.shared is not None:
+            self.shared.load(store, rt)
+
+    def forward(self, ctx, h, out, accumulate: bool = True) -> None:
+        k, T, E, top = ctx.rt.k, h.shape[0], self.n_experts, self.top
+        i32 = torch.int32
+        logits = ctx.ws.take((T, E), torch.float32)
+        k.gemm(h, self.w_router, logits, None, MODE_STORE_F32)
+        chosen, weights = ctx.ws.take((T, top), i32), ctx.ws.take((T, top), torch.float32)
+        k.route_topk(logits, top, chosen, weights)
+        P = T * top
+        max_tiles = k.route_max_tiles(P, E)
+        pairs, tokens = ctx.ws.take((P,), i32), ctx.ws.take((P,), i32)
+        tiles, n_tiles = ctx.ws.take((3 * max_tiles,), i32), ctx.ws.take((1,), i32)
+        k.route_sort(chosen, E, pairs, tokens, tiles, n_tiles)
+        act = ctx.ws.take((P, self.ff), ctx.rt.dtype)
+        k.grouped_gemm(h, self.w_gate_up, act, x_group_stride=0, out_group_stride=0, glu=(self.limit, self.alpha),
+                       routed=(tiles, n_tiles, max_tiles, tokens, pairs), rows=P)
+        rows = ctx.ws.take((P, self.hidden), torch.float32)
+        k.grouped_gemm(act, self.w_down, rows, x_group_stride=0, out_group_stride=0,
+                       routed=(tiles, n_tiles, max_tiles, pairs, pairs), rows=P)
+        k.route_combine(rows, weights, out, accumulate)
+        if self.shared is not None:
+            self.shared.forward(ctx, h, out)
+
+
+register_feed_forward("routed_experts", RoutedExperts)
