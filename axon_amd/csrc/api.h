@@ -239,21 +239,24 @@ int axk_route_combine(const float* rows, const float* weights, float* y, int n_t
                       void* stream);
 
 // A short causal convolution per channel and a gated linear recurrence (csrc/recurrent.hip).  A
-// request's state row (float32, rows state_stride apart) is [channels] of recurrent state, then
-// [taps - 1][channels] of the convolution's last inputs, oldest first; zeros for a new request.
+// request's state row (float32, rows state_stride apart) holds two copies of ([channels] of
+// recurrent state, then [taps - 1][channels] of the convolution's last inputs, oldest first); zeros
+// for a new request.  The state behind position p is in copy p & 1, so a step of one token reads one
+// copy and writes the other, and gives the same result if it is run again.
 // axk_causal_conv: u[t, c] = bias[c] + sum_k w[c, k] in(t - (taps - 1 - k)), inputs before the
-// step from the state (state_offset: where the kept inputs start in a row).  Reads the state only.
+// step from the state.  Reads the state only.
 // axk_gated_scan: per request of the step (spans [n][3] = (slot, first token, tokens); null: each
 // token a request of its own in slot seq_rows[t]) and channel, over its tokens in order:
 // r = sigmoid(gates r), i = sigmoid(gates i), a = exp(-decay r softplus(lam)),
 // S = a S + sqrt(1 - a^2) (i u), out = S gelu(y); then the state row is brought up to date
 // (S, and the convolution's inputs from x).  gates [T, channels / block_width, 2 block_width].
 int axk_causal_conv(const void* x, long x_stride, const void* w, const void* bias, int bias_is_f32, const float* state,
-                    long state_stride, int state_offset, const int32_t* seq_rows, float* u, int n_tokens, int channels,
-                    int taps, void* stream);
+                    long state_stride, const int32_t* positions, const int32_t* seq_rows, float* u, int n_tokens,
+                    int channels, int taps, void* stream);
 int axk_gated_scan(const float* gates, const float* u, const void* y, long y_stride, const void* x, long x_stride,
                    const void* lam, int lam_is_f32, float decay, float* state, long state_stride, const int32_t* spans,
-                   int n_spans, const int32_t* seq_rows, void* out, int channels, int block_width, int taps, void* stream);
+                   int n_spans, const int32_t* positions, const int32_t* seq_rows, void* out, int channels, int block_width,
+                   int taps, void* stream);
 
 // Attention over a latent cache (csrc/latent_attention.hip); a page is [page_size][rank + rot] elem.
 // axk_latent_prepare: from the float32 rows of the down projections, the normed query latent

@@ -1,11 +1,14 @@
 // A gated linear recurrence with a short causal convolution in front of it (the recurrent block of
 // Griffin-like models): per-request state in 32-bit floats, carried from step to step.
 //
-// A request's state row is [channels] of recurrent state followed by [taps - 1][channels] of the
-// convolution's last inputs (oldest first); a new request starts from zeros, which is also what
-// the convolution reads before the first token.  The tokens of a request are contiguous in a step
-// and a request is in a step once, so two tokens belong to one request iff their state slots
-// (seq_rows) are equal.
+// A request's state row holds two copies of ([channels] of recurrent state, then [taps - 1][channels]
+// of the convolution's last inputs, oldest first); a new request starts from zeros, which is also
+// what the convolution reads before the first token.  The state behind position p lives in copy
+// p & 1: a step whose first position is s reads copy (s - 1) & 1 and writes the copy of its last
+// position.  A step of one token therefore never writes what it read, and running it again (a
+// decoding step is run once before it is captured into a graph) gives the same state and the same
+// output.  The tokens of a request are contiguous in a step and a request is in a step once, so
+// two tokens belong to one request iff their state slots (seq_rows) are equal.
 #include "api.h"
 #include "common.h"
 
@@ -15,8 +18,8 @@ namespace {
 // token's.  One thread per (token, channel); inputs before the step come from the state.
 __global__ void causal_conv_kernel(const elem_t* __restrict__ x, long x_stride, const elem_t* __restrict__ w,
                                    const void* __restrict__ bias, int bias_is_f32, const float* __restrict__ state,
-                                   long state_stride, int state_offset, const int32_t* __restrict__ seq_rows,
-                                   float* __restrict__ u, int channels, int taps) {
+                                   long state_stride, const int32_t* __restrict__ positions,
+                                   const int32_t* __restrict__ seq_rows, float* __restrict__ u, int channels, int taps) {
   const int t = blockIdx.y;
   const int c = blockIdx.x * blockDim.x + threadIdx.x;
   if (c >= channels) return;
@@ -24,7 +27,9 @@ __global__ void causal_conv_kernel(const elem_t* __restrict__ x, long x_stride, 
   // how many earlier tokens of this step belong to the same request (up to taps - 1 matter)
   int inside = 0;
   while (inside < taps - 1 && t - inside - 1 >= 0 && seq_rows[t - inside - 1] == slot) ++inside;
-  const float* kept = state + (long)slot * state_stride + state_offset;      // [taps - 1][channels]
+  // the copy behind the position before the request's first of this step (not needed where all taps lie inside the step)
+  const int before = (positions[t] - inside + 1) & 1;
+  const float* kept = state + (long)slot * state_stride + (long)before * taps * channels + channels;      // [taps - 1][channels]
   float acc = 0.0f;
   for (int k = 0; k < taps; ++k) {
     const int back = taps - 1 - k;            // the input `back` tokens before this one
@@ -54,8 +59,9 @@ __device__ inline float gelu_tanh32(float z) {
 __global__ void gated_scan_kernel(const float* __restrict__ gates, const float* __restrict__ u,
                                   const elem_t* __restrict__ y, long y_stride, const elem_t* __restrict__ x, long x_stride,
                                   const void* __restrict__ lam, int lam_is_f32, float decay, float* __restrict__ state,
-                                  long state_stride, const int32_t* __restrict__ spans, const int32_t* __restrict__ seq_rows,
-                                  elem_t* __restrict__ out, int channels, int block_width, int taps) {
+                                  long state_stride, const int32_t* __restrict__ spans, const int32_t* __restrict__ positions,
+                                  const int32_t* __restrict__ seq_rows, elem_t* __restrict__ out, int channels, int block_width,
+                                  int taps) {
   const int c = blockIdx.x * blockDim.x + threadIdx.x;
   if (c >= channels) return;
   int slot, first, count;
@@ -69,8 +75,10 @@ __global__ void gated_scan_kernel(const float* __restrict__ gates, const float* 
   const float rate = -decay * softplus;
   const int b = c / block_width, j = c % block_width;
   const long gate_at = (long)b * 2 * block_width + j;
-  float* row = state + (long)slot * state_stride;
-  float S = row[c];
+  const int start = positions[first];
+  const float* from = state + (long)slot * state_stride + (long)((start + 1) & 1) * taps * channels;
+  float* row = state + (long)slot * state_stride + (long)((start + count - 1) & 1) * taps * channels;
+  float S = from[c];
   for (int t = first; t < first + count; ++t) {
     const float* g = gates + (long)t * 2 * channels + gate_at;
     const float r = sigmoid32(g[0]), i = sigmoid32(g[block_width]);
@@ -82,11 +90,12 @@ __global__ void gated_scan_kernel(const float* __restrict__ gates, const float* 
   }
   row[c] = S;
   // the convolution's last taps - 1 inputs: of (what was kept, this step's inputs) the last taps - 1;
-  // place i takes what lies `count` places later, read before it is written (ascending)
+  // place i takes what lies `count` places later (where both copies are one: read before it is written, ascending)
   float* kept = row + channels;
+  const float* kept_from = from + channels;
   for (int i = 0; i < taps - 1; ++i) {
     const int at = i + count;
-    kept[(long)i * channels + c] = at < taps - 1 ? kept[(long)at * channels + c]
+    kept[(long)i * channels + c] = at < taps - 1 ? kept_from[(long)at * channels + c]
                                                  : to_float(x[(long)(first + at - (taps - 1)) * x_stride + c]);
   }
 }
@@ -94,37 +103,36 @@ __global__ void gated_scan_kernel(const float* __restrict__ gates, const float* 
 }  // namespace
 
 extern "C" int axk_causal_conv(const void* x, long x_stride, const void* w, const void* bias, int bias_is_f32,
-                               const float* state, long state_stride, int state_offset, const int32_t* seq_rows, float* u,
-                               int n_tokens, int channels, int taps, void* stream) {
+                               const float* state, long state_stride, const int32_t* positions, const int32_t* seq_rows,
+                               float* u, int n_tokens, int channels, int taps, void* stream) {
   AXK_REQUIRE(n_tokens >= 0 && channels > 0 && taps >= 1 && x_stride >= channels,
               "causal_conv: bad sizes T=%d channels=%d taps=%d row stride %ld", n_tokens, channels, taps, x_stride);
-  AXK_REQUIRE(state_stride >= state_offset + (long)(taps - 1) * channels && state_offset >= 0,
-              "causal_conv: a state row of %ld floats does not hold %d x %d inputs from %d", state_stride, taps - 1, channels,
-              state_offset);
+  AXK_REQUIRE(state_stride >= 2L * taps * channels, "causal_conv: a state row of %ld floats does not hold 2 x %d x %d",
+              state_stride, taps, channels);
   AXK_REQUIRE(n_tokens <= 65535, "causal_conv: %d tokens in one step (at most 65535)", n_tokens);
   if (n_tokens == 0) return 0;
   dim3 grid(ceil_div(channels, 256), n_tokens);
   causal_conv_kernel<<<grid, 256, 0, (hipStream_t)stream>>>((const elem_t*)x, x_stride, (const elem_t*)w, bias, bias_is_f32,
-                                                           state, state_stride, state_offset, seq_rows, u, channels, taps);
+                                                           state, state_stride, positions, seq_rows, u, channels, taps);
   AXK_LAUNCH_CHECK("causal_conv");
   return 0;
 }
 
 extern "C" int axk_gated_scan(const float* gates, const float* u, const void* y, long y_stride, const void* x, long x_stride,
                               const void* lam, int lam_is_f32, float decay, float* state, long state_stride,
-                              const int32_t* spans, int n_spans, const int32_t* seq_rows, void* out, int channels,
-                              int block_width, int taps, void* stream) {
+                              const int32_t* spans, int n_spans, const int32_t* positions, const int32_t* seq_rows, void* out,
+                              int channels, int block_width, int taps, void* stream) {
   AXK_REQUIRE(n_spans >= 0 && channels > 0 && block_width > 0 && channels % block_width == 0 && taps >= 1,
               "gated_scan: bad sizes spans=%d channels=%d block width=%d taps=%d", n_spans, channels, block_width, taps);
-  AXK_REQUIRE(state_stride >= (long)taps * channels, "gated_scan: a state row of %ld floats does not hold %d x %d",
+  AXK_REQUIRE(state_stride >= 2L * taps * channels, "gated_scan: a state row of %ld floats does not hold 2 x %d x %d",
               state_stride, taps, channels);
-  AXK_REQUIRE(spans != nullptr || seq_rows != nullptr, "gated_scan: neither spans nor slots");
+  AXK_REQUIRE((spans != nullptr || seq_rows != nullptr) && positions != nullptr, "gated_scan: neither spans nor slots, or no positions");
   AXK_REQUIRE(n_spans <= 65535, "gated_scan: %d requests in one step (at most 65535)", n_spans);
   if (n_spans == 0) return 0;
   dim3 grid(ceil_div(channels, 64), n_spans);
   gated_scan_kernel<<<grid, 64, 0, (hipStream_t)stream>>>(gates, u, (const elem_t*)y, y_stride, (const elem_t*)x, x_stride, lam,
-                                                         lam_is_f32, decay, state, state_stride, spans, seq_rows,
-                                                         (elem_t*)out, channels, block_width, taps);
+                                                         lam_is_f32, decay, state, state_stride, spans, positions,
+                                                         seq_rows, (elem_t*)out, channels, block_width, taps);
   AXK_LAUNCH_CHECK("gated_scan");
   return 0;
 }

@@ -86,10 +86,10 @@ _SIGNATURES = {
     "axk_route_max_tiles": [c_int, c_int],
     "axk_route_sort": [c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p],
     "axk_route_combine": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
-    "axk_causal_conv": [c_void_p, c_long, c_void_p, c_void_p, c_int, c_void_p, c_long, c_int, c_void_p, c_void_p, c_int, c_int,
+    "axk_causal_conv": [c_void_p, c_long, c_void_p, c_void_p, c_int, c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_int, c_int,
                         c_int, c_void_p],
     "axk_gated_scan": [c_void_p, c_void_p, c_void_p, c_long, c_void_p, c_long, c_void_p, c_int, c_float, c_void_p, c_long,
-                       c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],
+                       c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],
     "axk_latent_prepare": [c_void_p, c_long, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_int, c_void_p, c_int, c_float,
                            c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_int, c_void_p],
     "axk_latent_query_rope": [c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],
@@ -755,29 +755,30 @@ class Kernels:
         return y
 
     # ------------------------------------------------------------------ convolution and recurrence with per-request state
-    def causal_conv(self, x: torch.Tensor, w: torch.Tensor, bias, state: torch.Tensor, state_offset: int, seq_rows: torch.Tensor,
-                    u: torch.Tensor) -> torch.Tensor:
+    def causal_conv(self, x: torch.Tensor, w: torch.Tensor, bias, state: torch.Tensor, positions: torch.Tensor,
+                    seq_rows: torch.Tensor, u: torch.Tensor) -> torch.Tensor:
         """u[t, c] = bias[c] + sum_k w[c, k] x(t - (taps - 1 - k)); x [T, C] in the compute dtype (rows may
-        be strided), inputs before the step from the float32 state rows [slots, >= offset + (taps - 1) C]."""
+        be strided), inputs before the step from the float32 state rows [slots, >= 2 taps C] (two copies,
+        the one behind position p at p & 1: see csrc/recurrent.hip)."""
         self._elem(x, "conv x"); self._elem(w, "conv w"); self._f32(state, "conv state"); self._f32(u, "conv u")
-        self._i32(seq_rows, "seq_rows")
+        self._i32(seq_rows, "seq_rows"); self._i32(positions, "positions")
         T, C = u.shape
         if x.shape != (T, C) or x.stride(1) != 1 or w.dim() != 2 or w.shape[0] != C or not w.is_contiguous() or seq_rows.numel() != T:
             raise KernelError(f"causal_conv: x {tuple(x.shape)}, w {tuple(w.shape)}, u {tuple(u.shape)}")
         if bias is not None and bias.numel() != C:
             raise KernelError(f"causal_conv: a bias of {bias.numel()} for {C} channels")
         self._check(self.lib.axk_causal_conv(_ptr(x), x.stride(0), _ptr(w), _ptr(bias), self._vec_flag(bias, "conv bias"),
-                                             _ptr(state), state.stride(0), int(state_offset), _ptr(seq_rows), _ptr(u), T, C,
+                                             _ptr(state), state.stride(0), _ptr(positions), _ptr(seq_rows), _ptr(u), T, C,
                                              w.shape[1], _stream()))
         return u
 
-    def gated_scan(self, gates, u, y, x, lam, decay: float, state, spans, seq_rows, out, block_width: int, taps: int):
+    def gated_scan(self, gates, u, y, x, lam, decay: float, state, spans, positions, seq_rows, out, block_width: int, taps: int):
         """The gated linear recurrence over each request's tokens (see csrc/recurrent.hip): gates
         [T, C / block_width, 2 block_width] and u [T, C] float32; y, x [T, C] compute dtype (rows may be
-        strided); state float32 [slots, >= taps C]; spans int32 [n, 3] = (slot, first token, tokens) or
+        strided); state float32 [slots, >= 2 taps C]; spans int32 [n, 3] = (slot, first token, tokens) or
         None (each token a request of its own in slot seq_rows[t]); out [T, C] compute dtype."""
         self._f32(gates, "scan gates"); self._f32(u, "scan u"); self._elem(y, "scan y"); self._elem(x, "scan x")
-        self._f32(state, "scan state"); self._elem(out, "scan out"); self._i32(seq_rows, "seq_rows")
+        self._f32(state, "scan state"); self._elem(out, "scan out"); self._i32(seq_rows, "seq_rows"); self._i32(positions, "positions")
         T, C = u.shape
         if (gates.shape != (T, 2 * C) and gates.numel() != T * 2 * C) or y.shape != (T, C) or x.shape != (T, C) or out.shape != (T, C) \
                 or y.stride(1) != 1 or x.stride(1) != 1 or not out.is_contiguous() or lam.numel() != C or seq_rows.numel() != T:
@@ -789,7 +790,8 @@ class Kernels:
             n = T
         self._check(self.lib.axk_gated_scan(_ptr(gates), _ptr(u), _ptr(y), y.stride(0), _ptr(x), x.stride(0), _ptr(lam),
                                             self._vec_flag(lam, "scan lam"), float(decay), _ptr(state), state.stride(0),
-                                            _ptr(spans), n, _ptr(seq_rows), _ptr(out), C, int(block_width), int(taps), _stream()))
+                                            _ptr(spans), n, _ptr(positions), _ptr(seq_rows), _ptr(out), C, int(block_width),
+                                            int(taps), _stream()))
         return out
 
     # ------------------------------------------------------------------ attention over a latent cache

@@ -6,7 +6,9 @@ causal convolution of `conv` taps per channel.  The channels form `blocks` equal
 the gates are r = sigmoid(Ra[b] u_b + ra[b]) and i = sigmoid(Ri[b] u_b + ri[b]).  Then
 a = exp(-decay * r * softplus(lam)), S_t = a S_(t-1) + sqrt(1 - a^2) (i u) from S = 0, and the
 output is Wo (S * y).  Gates, decays and the state are 32-bit; a request's state row holds S and
-the convolution's last conv - 1 inputs.
+the convolution's last conv - 1 inputs, twice: the state behind position p in copy p & 1, so that a
+decoding step reads one copy and writes the other and may be run again (the engine runs a step once
+before it captures it into a graph) with the same result.
 
 Parameters: `hidden_size`, `width`, `blocks`, `conv`, `decay` (default 8), `names` (the tensors'
 names under the prefix: scope "mix.", y, x, conv, ra, ri, lam, o; a bias is the name + ".b").
@@ -63,7 +65,7 @@ class GatedRecurrence(Mixer):
                 TensorDecl(n["lam"], (W,), "bias"), TensorDecl(n["o"], (self.hidden, W))]
 
     def state_spec(self) -> StateSpec:
-        return StateSpec(self.taps * self.width)
+        return StateSpec(2 * self.taps * self.width)
 
     def load(self, store, rt) -> None:
         n = self.n
@@ -91,11 +93,12 @@ class GatedRecurrence(Mixer):
         k.gemm(h, self.w_yx, yx, self.b_yx, MODE_STORE)
         y, x = yx[:, :C], yx[:, C:]
         u = ctx.ws.take((T, C), torch.float32)
-        k.causal_conv(x, self.conv_w, self.conv_b, state, C, ctx.seq_rows, u)
+        k.causal_conv(x, self.conv_w, self.conv_b, state, ctx.positions, ctx.seq_rows, u)
         gates = ctx.ws.take((T, 2 * C), torch.float32)
         k.grouped_gemm(u, self.w_gates, gates, x_group_stride=self.bw, out_group_stride=2 * self.bw, bias=self.b_gates)
         mixed = ctx.ws.take((T, C), ctx.rt.dtype)
-        k.gated_scan(gates, u, y, x, self.lam, self.decay, state, step_spans(ctx), ctx.seq_rows, mixed, self.bw, self.taps)
+        k.gated_scan(gates, u, y, x, self.lam, self.decay, state, step_spans(ctx), ctx.positions, ctx.seq_rows, mixed, self.bw,
+                     self.taps)
         k.gemm(mixed, self.w_o, out, None, MODE_ADD_F32 if accumulate else MODE_STORE_F32)
 
 

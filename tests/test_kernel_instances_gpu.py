@@ -228,6 +228,24 @@ def check_rmsnorm(dtype, dim):
 # --------------------------------------------------------------------------- the cases
 # (names of the instances the case is meant to select, the check, its arguments)
 BF, F32 = "bfloat16", "float32"
+def check_grouped(dtype, M, G, N, K, glu):
+    """A block-diagonal grouped product (gated or plain) against float64."""
+    k = kernels(dtype)
+    td = torch.bfloat16 if dtype == "bfloat16" else torch.float32
+    x = rnd(M, G * K, seed=4).to(torch.bfloat16).float()
+    w = rnd(G, (2 if glu else 1) * N, K, seed=5, scale=0.3).to(torch.bfloat16).float()
+    out = torch.zeros(M, G * N, dtype=torch.float32, device="cuda")
+    hit = launched(k, dtype, lambda: k.grouped_gemm(x.to(td).cuda(), w.to(td).cuda(), out, x_group_stride=K, out_group_stride=N,
+                                                    glu=(1.0, 1.702) if glu else None))
+    for g in range(G):
+        z = x[:, g * K:(g + 1) * K].double() @ w[g].double().T
+        if glu:
+            gate, up = torch.clamp(z[:, :N], max=1.0), torch.clamp(z[:, N:], -1.0, 1.0)
+            z = gate * torch.sigmoid(1.702 * gate) * (up + 1)
+        assert float((out[:, g * N:(g + 1) * N].cpu() - z.float()).abs().max()) <= tol(dtype, z.float(), bf16=1e-4)
+    return hit
+
+
 CASES = [
     # 32-bit FMA products: the float32 build's, and the bfloat16 build's for what cannot be packed
     (F32, ["gemm_fma<16,0>"], check_gemm, (F32, 5, 100, 70, MODE_STORE_F32, True)),
@@ -360,6 +378,13 @@ CASES = [
     (BF, ["gemm_tile<128,128,2,2,0,4>", "gemm_split_reduce<1>"], check_then_norm, (150, 256, 1024)),
     (BF, ["gemm_tile<256,256,4,2,1,2>"], check_gemm, (BF, 200, 18944, 3584, MODE_SWIGLU)),              # a 7B layer's at 200 rows
     (BF, ["gemm_tile<256,256,4,2,0,2>", "gemm_split_reduce<2>"], check_qkv_rope, (2048, 28, 4, 128, 3584, 64)),
+    # grouped products: (matrix cores or 32-bit FMA, gated epilogue)
+    (BF, ["grouped_gemm<1,0>"], check_grouped, (BF, 50, 3, 40, 64, False)),
+    (BF, ["grouped_gemm<1,1>"], check_grouped, (BF, 19, 2, 72, 160, True)),
+    (BF, ["grouped_gemm<0,0>"], check_grouped, (BF, 50, 3, 40, 24, False)),
+    (BF, ["grouped_gemm<0,1>"], check_grouped, (BF, 19, 2, 72, 40, True)),
+    (F32, ["grouped_gemm<0,0>"], check_grouped, (F32, 50, 3, 40, 64, False)),
+    (F32, ["grouped_gemm<0,1>"], check_grouped, (F32, 19, 2, 72, 160, True)),
     # attention on the matrix cores: (head size, query heads a block, pages of 64 positions or more)
     # and (head size, waves a block) (one wave a block in the decoding kernel up to 2,560 blocks of
     # positions, four beyond; two heads a block in the prompt kernel where tiles x heads are more
