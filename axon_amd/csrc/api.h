@@ -250,15 +250,20 @@ int axk_route_combine(const float* rows, const float* weights, float* y, int n_t
 // r = sigmoid(gates r), i = sigmoid(gates i), a = exp(-decay r softplus(lam)),
 // S = a S + sqrt(1 - a^2) (i u), out = S gelu(y); then the state row is brought up to date
 // (S, and the convolution's inputs from x).  gates [T, channels / block_width, 2 block_width].
+// terms (float32 [n_tokens, 3, channels], with spans): what does not depend on the state is worked
+// out for all tokens at once first, and the walk over a request's tokens is left with one
+// multiply-add a step (the same bits; for long stretches of tokens).
 int axk_causal_conv(const void* x, long x_stride, const void* w, const void* bias, int bias_is_f32, const float* state,
                     long state_stride, const int32_t* positions, const int32_t* seq_rows, float* u, int n_tokens,
                     int channels, int taps, void* stream);
 int axk_gated_scan(const float* gates, const float* u, const void* y, long y_stride, const void* x, long x_stride,
                    const void* lam, int lam_is_f32, float decay, float* state, long state_stride, const int32_t* spans,
                    int n_spans, const int32_t* positions, const int32_t* seq_rows, void* out, int channels, int block_width,
-                   int taps, void* stream);
+                   int taps, float* terms, int n_tokens, void* stream);
 
-// Attention over a latent cache (csrc/latent_attention.hip); a page is [page_size][rank + rot] elem.
+// Attention over a latent cache (csrc/latent_attention.hip); a page is [page_size][rank + rot] elem
+// (the latent and the rotated key part of each position), then [rank][page_size] (the latents again,
+// the positions of one dim side by side): 2 rank + rot elements a position.
 // axk_latent_prepare: from the float32 rows of the down projections, the normed query latent
 // (cq elem [T, q_rank]; q_rank 0: none) and, with write_kv, the normed key/value latent and the
 // rotated shared key part into the request's page.  axk_latent_query_rope: the rotated part of
@@ -271,6 +276,7 @@ int axk_latent_prepare(const float* fused, long stride, int q_at, int q_rank, in
                        int table_stride, void* cache, int page_size, void* cq, int n_tokens, int write_kv, void* stream);
 int axk_latent_query_rope(const float* q, int dim, int rot, int rot_dims, const float* table, float* q_full, int rank,
                           int heads, int n_tokens, void* stream);
+int axk_latent_attention_uses_mfma(int heads, int rank, int rot, int page_size);
 int axk_latent_attention(const float* q_full, const void* cache, const int32_t* block_table, int table_stride,
                          const int32_t* positions, const int32_t* seq_rows, float* o_lat, int n_tokens, int heads, int rank,
                          int rot, int page_size, int window, float scale, void* stream);

@@ -3,8 +3,11 @@
 // unrotated key is Wuk c and its value Wuv c; neither is ever built.  The query's unrotated part
 // is carried into the latent space instead (q_lat = Wuk^T q, a per-head product), so that
 //     score(i, j) = (q_lat_i . c_j + q_rot_i . k_rot_j) scale,      o_lat_i = sum_j p_ij c_j,
-// and the head's output is Wuv o_lat (another per-head product).  A page of the cache is
-// [page_size][rank + rot] in the compute dtype.  Scores, weights and sums are 32-bit.
+// and the head's output is Wuv o_lat (another per-head product).  A page of the cache holds its
+// positions twice: [page_size][rank + rot] rows (the latent and the rotated key part: what scores
+// read), then [rank][page_size], the latents again with the positions of one dim side by side
+// (what the matrix cores want as the operand of the weighted sum; the same layout as the values of
+// the grouped-query attention's pages).  Scores, weights and sums are 32-bit.
 #include "api.h"
 #include "common.h"
 
@@ -35,12 +38,17 @@ latent_prepare_kernel(const float* __restrict__ fused, long stride, int q_at, in
   if (!write_kv) return;
   const int pos = positions[t];
   const int page = block_table[(long)seq_rows[t] * table_stride + pos / page_size];
-  elem_t* dst = cache + ((long)page * page_size + pos % page_size) * (rank + rot);
+  elem_t* page_base = cache + (long)page * page_size * (2 * rank + rot);
+  elem_t* dst = page_base + (long)(pos % page_size) * (rank + rot);
+  elem_t* by_dim = page_base + (long)page_size * (rank + rot) + pos % page_size;      // [rank][page_size]
   float ss = 0.0f;
   for (int i = threadIdx.x; i < rank; i += 256) ss = fmaf(row[kv_at + i], row[kv_at + i], ss);
   const float inv = 1.0f / sqrtf(block_sum_256(ss, partial) / (float)rank + eps);
-  for (int i = threadIdx.x; i < rank; i += 256)
-    dst[i] = from_float((row[kv_at + i] * inv) * load_vec(kv_gain, kv_gain_is_f32, i));
+  for (int i = threadIdx.x; i < rank; i += 256) {
+    const elem_t v = from_float((row[kv_at + i] * inv) * load_vec(kv_gain, kv_gain_is_f32, i));
+    dst[i] = v;
+    by_dim[(long)i * page_size] = v;
+  }
   const float* kr = row + kv_at + rank;
   const int half = rot_dims / 2;
   const float* tab = table + (long)t * half * 2;
@@ -85,6 +93,7 @@ latent_attention_kernel(const float* __restrict__ q_full, const elem_t* __restri
   extern __shared__ float smem[];
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int width = rank + rot;
+  const long page_elems = (long)page_size * (width + rank);
   const long item = (long)blockIdx.x * LA_WAVES + wave;
   const bool active = item < (long)n_tokens * heads;
   const int t = active ? (int)(item / heads) : 0, h = active ? (int)(item % heads) : 0;
@@ -107,7 +116,7 @@ latent_attention_kernel(const float* __restrict__ q_full, const elem_t* __restri
     const bool seen = p >= lo && p <= pos;
     float s = -INFINITY;
     if (seen) {
-      const elem_t* key = cache + ((long)pages[p / page_size] * page_size + p % page_size) * width;
+      const elem_t* key = cache + (long)pages[p / page_size] * page_elems + (long)(p % page_size) * width;
       float dot = 0.0f;
       for (int i = 0; i < width; ++i) dot = fmaf(qs[i], to_float(key[i]), dot);
       s = dot * scale;
@@ -123,7 +132,7 @@ latent_attention_kernel(const float* __restrict__ q_full, const elem_t* __restri
     for (int j = j_lo; j <= j_hi; ++j) {
       const float wj = __shfl(w, j, 64);
       const int pj = b * 64 + j;
-      const elem_t* val = cache + ((long)pages[pj / page_size] * page_size + pj % page_size) * width;
+      const elem_t* val = cache + (long)pages[pj / page_size] * page_elems + (long)(pj % page_size) * width;
 #pragma unroll
       for (int i = 0; i < MAX_OWN; ++i) {
         const int d = lane + 64 * i;
@@ -140,7 +149,147 @@ latent_attention_kernel(const float* __restrict__ q_full, const elem_t* __restri
   }
 }
 
+#if AXON_BF16
+typedef __attribute__((ext_vector_type(8))) __bf16 la_bf16x8;
+typedef __attribute__((ext_vector_type(4))) float la_f32x4;
+__device__ inline la_bf16x8 la_frag(uint4 v) { return __builtin_bit_cast(la_bf16x8, v); }
+
+// The same attention on the matrix cores.  One wave per (token, sixteen heads), four waves a block,
+// each on its own: the sixteen heads of a token see the same positions, so a block of 64 positions is
+//   S^T [position, head] = K [position, dims] Q^T           (rank + rot dims in chunks of 32),
+//   a maximum, weights and their sum per head (a lane holds 16 positions of its head; the four
+//   lanes of a head meet by lane permutation), the running (m, l) and O^T rescaled, then
+//   O^T [dim, head] += C^T [dim, position] P^T              (positions in two chunks of 32),
+// with K rows and the rows of C^T straight from the page into the first operand (16 or 8 bytes a
+// lane) and the rounded weights, as they lie in the accumulators, as the second.  RT: tiles of 16
+// latent dims at most; QC: chunks of 32 key dims at most.  Pages hold a multiple of 64 positions.
+template <int RT, int QC>
+__global__ void __launch_bounds__(256)
+latent_attention_mfma_kernel(const float* __restrict__ q_full, const bf16_t* __restrict__ cache,
+                             const int32_t* __restrict__ block_table, int table_stride, const int32_t* __restrict__ positions,
+                             const int32_t* __restrict__ seq_rows, float* __restrict__ o_lat, int n_tokens, int heads, int rank,
+                             int rot, int page_size, int window, float scale) {
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int groups = heads / 16;
+  const long item = (long)blockIdx.x * 4 + wave;
+  if (item >= (long)n_tokens * groups) return;
+  const int t = (int)(item / groups), hg = (int)(item % groups);
+  const int width = rank + rot, qc = width / 32, rt = rank / 16;
+  const int j = lane & 15, g = lane >> 4;
+  const float* qrow = q_full + ((long)t * heads + hg * 16 + j) * width + 8 * g;
+  uint4 qf[QC];
+#pragma unroll
+  for (int kc = 0; kc < QC; ++kc) {
+    if (kc < qc) {
+      const float4 a = *reinterpret_cast<const float4*>(qrow + 32 * kc), b = *reinterpret_cast<const float4*>(qrow + 32 * kc + 4);
+      qf[kc] = make_uint4(pack2_bf16(a.x, a.y), pack2_bf16(a.z, a.w), pack2_bf16(b.x, b.y), pack2_bf16(b.z, b.w));
+    } else {
+      qf[kc] = make_uint4(0, 0, 0, 0);
+    }
+  }
+  const int pos = positions[t];
+  const int lo = window > 0 ? max(0, pos + 1 - window) : 0;
+  const int32_t* pages = block_table + (long)seq_rows[t] * table_stride;
+  const long page_elems = (long)page_size * (width + rank);
+  la_f32x4 acc[RT];
+#pragma unroll
+  for (int i = 0; i < RT; ++i) acc[i] = la_f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+  float m = -INFINITY, l = 0.0f;
+  for (int b = lo / 64; b <= pos / 64; ++b) {
+    const int p0 = b * 64, in0 = p0 % page_size;
+    const bf16_t* page = cache + (long)pages[p0 / page_size] * page_elems;
+    const bf16_t* kbase = page + (long)in0 * width + 8 * g;
+    const bf16_t* vbase = page + (long)page_size * width + in0 + 4 * g;
+    la_f32x4 s[4];
+#pragma unroll
+    for (int pt = 0; pt < 4; ++pt) {
+      s[pt] = la_f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+      const bf16_t* krow = kbase + (long)(16 * pt + j) * width;
+#pragma unroll
+      for (int kc = 0; kc < QC; ++kc)
+        if (kc < qc)
+          s[pt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(la_frag(*reinterpret_cast<const uint4*>(krow + 32 * kc)),
+                                                          la_frag(qf[kc]), s[pt], 0, 0, 0);
+    }
+    float mx = -INFINITY;
+#pragma unroll
+    for (int pt = 0; pt < 4; ++pt)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int p = p0 + 16 * pt + 4 * g + i;
+        const float v = (p >= lo && p <= pos) ? s[pt][i] * scale : -INFINITY;
+        s[pt][i] = v;
+        mx = fmaxf(mx, v);
+      }
+    mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+    const float m_new = fmaxf(m, mx);
+    const float fold = expf(m - m_new);
+    float sum = 0.0f;
+#pragma unroll
+    for (int pt = 0; pt < 4; ++pt)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const float w = expf(s[pt][i] - m_new);        // 0 where the position is not seen
+        s[pt][i] = w;
+        sum += w;
+      }
+    sum += __shfl_xor(sum, 16, 64);
+    sum += __shfl_xor(sum, 32, 64);
+    l = fmaf(l, fold, sum);
+    m = m_new;
+    uint4 pf[2];
+#pragma unroll
+    for (int c = 0; c < 2; ++c)
+      pf[c] = make_uint4(pack2_bf16(s[2 * c][0], s[2 * c][1]), pack2_bf16(s[2 * c][2], s[2 * c][3]),
+                         pack2_bf16(s[2 * c + 1][0], s[2 * c + 1][1]), pack2_bf16(s[2 * c + 1][2], s[2 * c + 1][3]));
+#pragma unroll
+    for (int dt = 0; dt < RT; ++dt) {
+      if (dt < rt) {
+        const bf16_t* vrow = vbase + (long)(16 * dt + j) * page_size;
+        uint2 v[4];
+#pragma unroll
+        for (int c = 0; c < 2; ++c) {
+          v[2 * c] = *reinterpret_cast<const uint2*>(vrow + 32 * c);
+          v[2 * c + 1] = *reinterpret_cast<const uint2*>(vrow + 32 * c + 16);
+        }
+        acc[dt] *= fold;
+#pragma unroll
+        for (int c = 0; c < 2; ++c)
+          acc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(la_frag(make_uint4(v[2 * c].x, v[2 * c].y, v[2 * c + 1].x, v[2 * c + 1].y)),
+                                                            la_frag(pf[c]), acc[dt], 0, 0, 0);
+      }
+    }
+  }
+  const float inv = 1.0f / l;
+  float* dst = o_lat + ((long)t * heads + hg * 16 + j) * rank + 4 * g;
+#pragma unroll
+  for (int dt = 0; dt < RT; ++dt)
+    if (dt < rt) *reinterpret_cast<float4*>(dst + 16 * dt) = make_float4(acc[dt][0] * inv, acc[dt][1] * inv, acc[dt][2] * inv, acc[dt][3] * inv);
+}
+
+template <int RT, int QC>
+static void launch_latent_mfma(const float* q_full, const void* cache, const int32_t* block_table, int table_stride,
+                               const int32_t* positions, const int32_t* seq_rows, float* o_lat, int n_tokens, int heads, int rank,
+                               int rot, int page_size, int window, float scale, hipStream_t stream) {
+  const long items = (long)n_tokens * (heads / 16);
+  latent_attention_mfma_kernel<RT, QC><<<(unsigned)((items + 3) / 4), 256, 0, stream>>>(
+      q_full, (const bf16_t*)cache, block_table, table_stride, positions, seq_rows, o_lat, n_tokens, heads, rank, rot, page_size,
+      window, scale);
+}
+#endif
+
 }  // namespace
+
+// 1 where axk_latent_attention runs on the matrix cores (the bfloat16 build, heads in sixteens,
+// a latent in sixteens up to 512, key rows in chunks of 32 up to 640, pages of a multiple of 64).
+extern "C" int axk_latent_attention_uses_mfma(int heads, int rank, int rot, int page_size) {
+#if AXON_BF16
+  return heads % 16 == 0 && rank % 16 == 0 && (rank + rot) % 32 == 0 && page_size % 64 == 0 && rank <= 512 && rank + rot <= 640;
+#else
+  return 0;
+#endif
+}
 
 extern "C" int axk_latent_prepare(const float* fused, long stride, int q_at, int q_rank, int kv_at, int rank, int rot,
                                   int rot_dims, const void* q_gain, int q_gain_is_f32, const void* kv_gain,
@@ -180,6 +329,23 @@ extern "C" int axk_latent_attention(const float* q_full, const void* cache, cons
   AXK_REQUIRE(rank <= 1024, "latent_attention: a latent of %d dims (at most 1024)", rank);
   AXK_REQUIRE((long)(rank + rot) * LA_WAVES * 4 <= 64 * 1024, "latent_attention: keys of %d dims do not fit LDS", rank + rot);
   if (n_tokens == 0) return 0;
+#if AXON_BF16
+  if (axk_latent_attention_uses_mfma(heads, rank, rot, page_size) && ((uintptr_t)q_full & 15) == 0 && ((uintptr_t)cache & 15) == 0 &&
+      ((uintptr_t)o_lat & 15) == 0) {
+    hipStream_t s = (hipStream_t)stream;
+    if (rank <= 64 && rank + rot <= 128)
+      launch_latent_mfma<4, 4>(q_full, cache, block_table, table_stride, positions, seq_rows, o_lat, n_tokens, heads, rank, rot,
+                               page_size, window, scale, s);
+    else if (rank <= 128 && rank + rot <= 256)
+      launch_latent_mfma<8, 8>(q_full, cache, block_table, table_stride, positions, seq_rows, o_lat, n_tokens, heads, rank, rot,
+                               page_size, window, scale, s);
+    else
+      launch_latent_mfma<32, 20>(q_full, cache, block_table, table_stride, positions, seq_rows, o_lat, n_tokens, heads, rank, rot,
+                                 page_size, window, scale, s);
+    AXK_LAUNCH_CHECK("latent_attention");
+    return 0;
+  }
+#endif
   const long items = (long)n_tokens * heads;
   const size_t lds = (size_t)(rank + rot) * LA_WAVES * sizeof(float);
   latent_attention_kernel<<<(unsigned)((items + LA_WAVES - 1) / LA_WAVES), LA_WAVES * 64, lds, (hipStream_t)stream>>>(

@@ -100,6 +100,71 @@ __global__ void gated_scan_kernel(const float* __restrict__ gates, const float* 
   }
 }
 
+// The same recurrence for long stretches of tokens, in two launches.  First, for every (token,
+// channel) at once, what does not depend on the state: a, b = (sqrt(1 - a^2) i) u and gelu(y), the
+// very operations of the kernel above, kept in 32-bit.  Then a thread per (request, channel) walks
+// S = a S + b with sixteen steps' operands asked for ahead of the chain that needs them.  The bits
+// are those of the kernel above.
+__global__ void gated_scan_terms_kernel(const float* __restrict__ gates, const float* __restrict__ u,
+                                        const elem_t* __restrict__ y, long y_stride, const void* __restrict__ lam,
+                                        int lam_is_f32, float decay, float* __restrict__ terms, int channels, int block_width) {
+  const int t = blockIdx.y;
+  const int c = blockIdx.x * blockDim.x + threadIdx.x;
+  if (c >= channels) return;
+  const float l = load_vec(lam, lam_is_f32, c);
+  const float softplus = l > 20.0f ? l : log1pf(expf(l));
+  const float rate = -decay * softplus;
+  const int b = c / block_width, j = c % block_width;
+  const float* g = gates + (long)t * 2 * channels + (long)b * 2 * block_width + j;
+  const float r = sigmoid32(g[0]), i = sigmoid32(g[block_width]);
+  const float log_a = rate * r;
+  const float mult = sqrtf(-expm1f(2.0f * log_a));
+  float* dst = terms + (long)t * 3 * channels + c;
+  dst[0] = expf(log_a);
+  dst[channels] = (mult * i) * u[(long)t * channels + c];
+  dst[2 * channels] = gelu_tanh32(to_float(y[(long)t * y_stride + c]));
+}
+
+#define SCAN_AHEAD 16
+__global__ void gated_scan_walk_kernel(const float* __restrict__ terms, const elem_t* __restrict__ x, long x_stride,
+                                       float* __restrict__ state, long state_stride, const int32_t* __restrict__ spans,
+                                       const int32_t* __restrict__ positions, elem_t* __restrict__ out, int channels, int taps) {
+  const int c = blockIdx.x * blockDim.x + threadIdx.x;
+  if (c >= channels) return;
+  const int slot = spans[3 * blockIdx.y], first = spans[3 * blockIdx.y + 1], count = spans[3 * blockIdx.y + 2];
+  const int start = positions[first];
+  const float* from = state + (long)slot * state_stride + (long)((start + 1) & 1) * taps * channels;
+  float* row = state + (long)slot * state_stride + (long)((start + count - 1) & 1) * taps * channels;
+  float S = from[c];
+  int t = first;
+  for (; t + SCAN_AHEAD <= first + count; t += SCAN_AHEAD) {
+    float a[SCAN_AHEAD], b[SCAN_AHEAD], gy[SCAN_AHEAD];
+#pragma unroll
+    for (int i = 0; i < SCAN_AHEAD; ++i) {
+      const float* src = terms + (long)(t + i) * 3 * channels + c;
+      a[i] = src[0]; b[i] = src[channels]; gy[i] = src[2 * channels];
+    }
+#pragma unroll
+    for (int i = 0; i < SCAN_AHEAD; ++i) {
+      S = fmaf(a[i], S, b[i]);
+      out[(long)(t + i) * channels + c] = from_float(S * gy[i]);
+    }
+  }
+  for (; t < first + count; ++t) {
+    const float* src = terms + (long)t * 3 * channels + c;
+    S = fmaf(src[0], S, src[channels]);
+    out[(long)t * channels + c] = from_float(S * src[2 * channels]);
+  }
+  row[c] = S;
+  float* kept = row + channels;
+  const float* kept_from = from + channels;
+  for (int i = 0; i < taps - 1; ++i) {
+    const int at = i + count;
+    kept[(long)i * channels + c] = at < taps - 1 ? kept_from[(long)at * channels + c]
+                                                 : to_float(x[(long)(first + at - (taps - 1)) * x_stride + c]);
+  }
+}
+
 }  // namespace
 
 extern "C" int axk_causal_conv(const void* x, long x_stride, const void* w, const void* bias, int bias_is_f32,
@@ -121,7 +186,7 @@ extern "C" int axk_causal_conv(const void* x, long x_stride, const void* w, cons
 extern "C" int axk_gated_scan(const float* gates, const float* u, const void* y, long y_stride, const void* x, long x_stride,
                               const void* lam, int lam_is_f32, float decay, float* state, long state_stride,
                               const int32_t* spans, int n_spans, const int32_t* positions, const int32_t* seq_rows, void* out,
-                              int channels, int block_width, int taps, void* stream) {
+                              int channels, int block_width, int taps, float* terms, int n_tokens, void* stream) {
   AXK_REQUIRE(n_spans >= 0 && channels > 0 && block_width > 0 && channels % block_width == 0 && taps >= 1,
               "gated_scan: bad sizes spans=%d channels=%d block width=%d taps=%d", n_spans, channels, block_width, taps);
   AXK_REQUIRE(state_stride >= 2L * taps * channels, "gated_scan: a state row of %ld floats does not hold 2 x %d x %d",
@@ -130,6 +195,16 @@ extern "C" int axk_gated_scan(const float* gates, const float* u, const void* y,
   AXK_REQUIRE(n_spans <= 65535, "gated_scan: %d requests in one step (at most 65535)", n_spans);
   if (n_spans == 0) return 0;
   dim3 grid(ceil_div(channels, 64), n_spans);
+  if (terms != nullptr && spans != nullptr && n_tokens > 0) {
+    AXK_REQUIRE(n_tokens <= 65535, "gated_scan: %d tokens in one step (at most 65535)", n_tokens);
+    dim3 wide(ceil_div(channels, 256), n_tokens);
+    gated_scan_terms_kernel<<<wide, 256, 0, (hipStream_t)stream>>>(gates, u, (const elem_t*)y, y_stride, lam, lam_is_f32, decay,
+                                                                  terms, channels, block_width);
+    gated_scan_walk_kernel<<<grid, 64, 0, (hipStream_t)stream>>>(terms, (const elem_t*)x, x_stride, state, state_stride, spans,
+                                                                positions, (elem_t*)out, channels, taps);
+    AXK_LAUNCH_CHECK("gated_scan");
+    return 0;
+  }
   gated_scan_kernel<<<grid, 64, 0, (hipStream_t)stream>>>(gates, u, (const elem_t*)y, y_stride, (const elem_t*)x, x_stride, lam,
                                                          lam_is_f32, decay, state, state_stride, spans, positions,
                                                          seq_rows, (elem_t*)out, channels, block_width, taps);

@@ -89,7 +89,7 @@ _SIGNATURES = {
     "axk_causal_conv": [c_void_p, c_long, c_void_p, c_void_p, c_int, c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_int, c_int,
                         c_int, c_void_p],
     "axk_gated_scan": [c_void_p, c_void_p, c_void_p, c_long, c_void_p, c_long, c_void_p, c_int, c_float, c_void_p, c_long,
-                       c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],
+                       c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_int, c_void_p],
     "axk_latent_prepare": [c_void_p, c_long, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_int, c_void_p, c_int, c_float,
                            c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_int, c_void_p],
     "axk_latent_query_rope": [c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],
@@ -206,7 +206,7 @@ class Kernels:
                   "fill_i32", "fill_f32", "call", "norm_add", "round_rows", "activation", "clamped_glu", "grouped_gemm",
                   "route_topk", "route_sort", "route_combine", "causal_conv", "gated_scan", "latent_prepare",
                   "latent_query_rope", "latent_attention")
-    _MATRIX_AT = {"gemm": 1, "gemm_qkv_rope": 1, "gemm_normed_glu": 3, "gemm_normed_qkv_rope": 3}   # which argument is W
+    _MATRIX_AT = {"gemm": 1, "gemm_qkv_rope": 1, "gemm_normed_glu": 3, "gemm_normed_qkv_rope": 3, "grouped_gemm": 1}   # which argument is W
 
     def set_launch_hook(self, hook) -> None:
         """`hook(name, matrix_bytes)` is told of every call that has launched kernels, with the
@@ -226,7 +226,7 @@ class Kernels:
                     w = a[self._MATRIX_AT[_name]]
                     data = w.data if isinstance(w, PackedMatrix) else w
                     nbytes = data.numel() * data.element_size()
-                    label = f"{_name} {w.shape[0]}x{w.shape[1]}"
+                    label = f"{_name} {'x'.join(str(n) for n in w.shape)}"
                 hook(label, nbytes)
                 return out
             self.__dict__[name] = told
@@ -783,15 +783,18 @@ class Kernels:
         if (gates.shape != (T, 2 * C) and gates.numel() != T * 2 * C) or y.shape != (T, C) or x.shape != (T, C) or out.shape != (T, C) \
                 or y.stride(1) != 1 or x.stride(1) != 1 or not out.is_contiguous() or lam.numel() != C or seq_rows.numel() != T:
             raise KernelError(f"gated_scan: gates {tuple(gates.shape)}, u {tuple(u.shape)}, y {tuple(y.shape)}, out {tuple(out.shape)}")
+        terms = None
         if spans is not None:
             self._i32(spans, "scan spans")
             n = spans.shape[0]
+            if T > 4 * n:            # stretches of tokens: the state-free terms for all tokens at once, then a lean walk
+                terms = torch.empty((T, 3, C), dtype=torch.float32, device=u.device)
         else:
             n = T
         self._check(self.lib.axk_gated_scan(_ptr(gates), _ptr(u), _ptr(y), y.stride(0), _ptr(x), x.stride(0), _ptr(lam),
                                             self._vec_flag(lam, "scan lam"), float(decay), _ptr(state), state.stride(0),
                                             _ptr(spans), n, _ptr(positions), _ptr(seq_rows), _ptr(out), C, int(block_width),
-                                            int(taps), _stream()))
+                                            int(taps), _ptr(terms), T, _stream()))
         return out
 
     # ------------------------------------------------------------------ attention over a latent cache
@@ -802,8 +805,8 @@ class Kernels:
         T = positions.numel()
         if fused.shape[0] != T or (rot_dims and table.shape != (T, rot_dims // 2, 2)) or seq_rows.numel() != T:
             raise KernelError(f"latent_prepare: fused {tuple(fused.shape)}, table {tuple(table.shape)} for {T} tokens")
-        if cache.dim() != 4 or tuple(cache.shape[1:]) != (1, page_size, rank + rot) or not cache.is_contiguous():
-            raise KernelError(f"latent_prepare: cache {tuple(cache.shape)} is not [pages, 1, {page_size}, {rank + rot}]")
+        if cache.dim() != 4 or tuple(cache.shape[1:]) != (1, page_size, 2 * rank + rot) or not cache.is_contiguous():
+            raise KernelError(f"latent_prepare: cache {tuple(cache.shape)} is not [pages, 1, {page_size}, {2 * rank + rot}]")
         if q_rank:
             self._elem(cq, "latent cq")
             if cq.shape != (T, q_rank) or not cq.is_contiguous() or q_gain.numel() != q_rank:
@@ -831,8 +834,8 @@ class Kernels:
         T = positions.numel()
         if q_full.shape != (T, heads * (rank + rot)) or o_lat.shape != (T, heads * rank) or seq_rows.numel() != T:
             raise KernelError(f"latent_attention: q_full {tuple(q_full.shape)}, o_lat {tuple(o_lat.shape)} for {T} tokens")
-        if cache.dim() != 4 or tuple(cache.shape[1:]) != (1, page_size, rank + rot) or not cache.is_contiguous():
-            raise KernelError(f"latent_attention: cache {tuple(cache.shape)} is not [pages, 1, {page_size}, {rank + rot}]")
+        if cache.dim() != 4 or tuple(cache.shape[1:]) != (1, page_size, 2 * rank + rot) or not cache.is_contiguous():
+            raise KernelError(f"latent_attention: cache {tuple(cache.shape)} is not [pages, 1, {page_size}, {2 * rank + rot}]")
         self._check(self.lib.axk_latent_attention(_ptr(q_full), _ptr(cache), _ptr(block_table), block_table.shape[-1],
                                                   _ptr(positions), _ptr(seq_rows), _ptr(o_lat), T, heads, rank, rot, page_size,
                                                   int(window), float(scale), _stream()))

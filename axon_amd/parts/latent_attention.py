@@ -6,8 +6,9 @@ and rot_dim more that are one rotated key part shared by all heads.  A head's un
 Wuk c and its value Wuv c; the score is (q_unrot . k_unrot + q_rot . k_rot) * scale over a
 causal window; the concatenated heads are multiplied by sigmoid(Wg h) and projected by Wo.
 
-Only c and the rotated key part are cached (one row of kv_rank + rot_dim per position), and the
-keys and values are never built: the unrotated query is carried into the latent space
+Only c and the rotated key part are cached, and the keys and values are never built (a position
+takes 2 kv_rank + rot_dim elements of its page: the row the scores read, and the latent once more
+with the positions of one dim side by side, as the matrix cores want the weighted sum's operand): the unrotated query is carried into the latent space
 (q_lat = Wuk^T q_unrot, a per-head product), attention runs there, and the head's output is
 Wuv (sum_j p_j c_j), a second per-head product.
 
@@ -60,7 +61,7 @@ class LatentAttention(Mixer):
         return t
 
     def cache_spec(self) -> Optional[CacheSpec]:
-        return CacheSpec(entries=1, heads=1, head_dim=self.kv_rank + self.rot, window=self.window)
+        return CacheSpec(entries=1, heads=1, head_dim=2 * self.kv_rank + self.rot, window=self.window)
 
     def load(self, store, rt) -> None:
         n, H = self.n, self.heads

@@ -86,8 +86,98 @@ def bandwidth(torch):
     return out
 
 
+# --design pikesun: layer sizes that resemble real models of that design (random weights), each beside
+# the dense Qwen2 decoder of the same width, depth and feed-forward work a token.  Every fourth layer's
+# pattern: recurrence + dense, latent attention + experts, recurrence + experts (shared tensors), latent
+# attention + experts.
+def _pikesun_sizes(width, rec_width, blocks, heads, q_rank, experts, top, expert_ff, shared_ff, dense_ff, window):
+    rec = {"type": "rglru", "mixer": {"width": rec_width, "blocks": blocks, "conv": 4}}
+    att = {"type": "latent_attention", "mixer": {"heads": heads, "dim": 128, "rot_dim": 64, "vdim": 128, "kv_rank": 512,
+                                                 "q_rank": q_rank, "rot": {"base": 10000.0, "dims": 64}, "scale": 192 ** -0.5,
+                                                 "mask": {"size": window}}}
+    moe = {"kind": "moe", "router": {"experts": experts, "top": top}, "expert": {"ff": expert_ff, "limit": 7.0},
+           "shared": {"ff": shared_ff, "limit": 7.0}}
+    layers = [dict(rec, mlp={"kind": "dense", "ff": dense_ff}), dict(att, mlp=moe), dict(rec, mlp=moe), dict(att, mlp=moe)]
+    return {"architecture": "Pikesun", "embedding": {"scale": 1.0}, "layers": layers, "norm": {"eps": 1e-6},
+            "residual_mult": 1.0, "vocab": 32000, "width": width}
+
+
+def _qwen_sizes(width, heads, kv_heads, ff):
+    return dict(architectures=["Qwen2ForCausalLM"], model_type="qwen2", num_hidden_layers=4, hidden_size=width,
+                intermediate_size=ff, num_attention_heads=heads, num_key_value_heads=kv_heads, head_dim=128, vocab_size=32000,
+                max_position_embeddings=8192, rope_theta=10000.0, rms_norm_eps=1e-6, tie_word_embeddings=False)
+
+
+DESIGN_SIZES = {
+    "2048": (_pikesun_sizes(2048, 2560, 10, 16, 768, 32, 4, 704, 1408, 5632, 1024), _qwen_sizes(2048, 16, 2, 5632)),
+    "4096": (_pikesun_sizes(4096, 5120, 20, 32, 1536, 64, 6, 1408, 2816, 11008, 2048), _qwen_sizes(4096, 32, 8, 11008)),
+}
+
+
+def design(args, torch) -> int:
+    """Prefill and decoding of the Pikesun design at sizes that resemble real models' layers, beside the
+    dense decoder of equal width: a prompt of --prompt tokens (default 2,048) in one step, decoding at
+    --batch (default 8) behind such prompts from graphs, and each kind of step kernel by kernel."""
+    import axon_amd
+    from axon_amd.engine import StepEntry
+    T, batch, steps = args.prompt or 2048, args.batch, args.steps or 64
+    out = {"design": "pikesun", "dtype": args.dtype, "prompt_tokens": T, "batch": batch, "data": "synthetic (random weights)",
+           "sizes": {}}
+    gen = torch.Generator().manual_seed(0)
+    for size, pair in DESIGN_SIZES.items():
+        if args.design_size and size != args.design_size:
+            continue
+        row = out["sizes"][size] = {}
+        for label, cfg in zip(("pikesun", "qwen2"), pair):
+            llm = axon_amd.load(cfg, dtype=args.dtype, random_seed=0, init_std=0.02, page_size=64,
+                                num_pages=(batch + 1) * (-(-(T + steps + args.warmup + 80) // 64)) + 8, max_seqs=batch + 1,
+                                max_batch_tokens=T, max_seq_len=T + steps + args.warmup + 80)
+            eng = llm.engine
+            V = llm.model.vocab_size
+            prompt = lambda n: torch.randint(0, V, (n,), generator=gen).tolist()
+            p = prompt(T)
+            eng.step([StepEntry("warm", p, [T - 1])], end=["warm"])
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(3):
+                eng.step([StepEntry("pf", p, [T - 1])], end=["pf"])
+            torch.cuda.synchronize()
+            pf = (time.perf_counter() - t0) / 3
+            kernels_pf, _ = eng.profile([StepEntry("pp", p, [T - 1])], end=["pp"])
+            ids = [f"d{i}" for i in range(batch)]
+            for rid in ids:
+                eng.step([StepEntry(rid, prompt(T), [])])
+            kernels_dec, _ = eng.profile([StepEntry(rid, prompt(1), [0]) for rid in ids])
+            eng.step([StepEntry(rid, prompt(1), [0]) for rid in ids])
+            pending = eng.picks_async()
+            for i in range(args.warmup + steps):
+                if i == args.warmup:
+                    pending.tolist()
+                    torch.cuda.synchronize()
+                    t0 = time.perf_counter()
+                eng.step_from_picks(ids)
+                behind = eng.picks_async()
+                pending.tolist()
+                pending = behind
+            pending.tolist()
+            torch.cuda.synchronize()
+            dec = (time.perf_counter() - t0) / steps
+            top = lambda rows: [{"kernel": r["name"], "us": round(r["ms"] * 1e3, 1), "launches": r["launches"]}
+                                for r in sorted(rows, key=lambda r: -r["ms"])[:14]]
+            row[label] = {"prefill_ms": round(pf * 1e3, 3), "prefill_tok_s": round(T / pf, 1), "decode_ms": round(dec * 1e3, 3),
+                          "decode_tok_s": round(batch / dec, 1), "prefill_kernels": top(kernels_pf), "decode_kernels": top(kernels_dec)}
+            eng.release_all()
+            del eng, llm
+            torch.cuda.empty_cache()
+    print(json.dumps(out))
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
+    ap.add_argument("--design", default="", choices=["", "pikesun"], help="instead of the headline benchmark: prefill and "
+                    "decoding of this design at sizes that resemble real models' layers, beside the dense decoder of equal size")
+    ap.add_argument("--design-size", default="", help="with --design: only this size (2048 or 4096)")
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=0, help="timed decode steps: every request generates this many tokens "
                     "(default: the size's own workload, 256 or 128)")
@@ -119,6 +209,8 @@ def main() -> int:
     if args.phase == "bandwidth":
         print(json.dumps(bandwidth(torch)))
         return 0
+    if args.design:
+        return design(args, torch)
 
     cfg = dict(SIZES[args.sizes])
     name = f"Qwen2.5-{args.sizes.upper()} sizes"

@@ -26,7 +26,7 @@ def test_config_json_selects_the_class_and_describes_the_layers():
     assert (m["window"], m["kv_rank"], m["rot_dim"], m["position"].params["theta"]) == (9, 20, 4, 100.0)
     model = build_model_description(c)
     plan = model.cache_plan
-    assert [(s.entries, s.heads, s.head_dim, s.window, n) for s, n in zip(plan.group_specs, plan.group_layers)] == [(1, 1, 24, 9, 2)]
+    assert [(s.entries, s.heads, s.head_dim, s.window, n) for s, n in zip(plan.group_specs, plan.group_layers)] == [(1, 1, 44, 9, 2)]
     assert plan.state_elems == [(2 * 3 * 72, "float32")] * 2
     assert [(b.group, b.index, b.state_index) for b in plan.bindings] == [(0, 0, -1), (-1, -1, 0), (-1, -1, 1), (0, 1, -1)]
 
@@ -40,7 +40,7 @@ def test_the_declared_tensors_are_the_checkpoints(name):
 
 def test_two_attention_layers_of_other_sizes_get_pools_of_their_own():
     plan = build_model_description(config_from_dict(MODELS["R"]["cfg"])).cache_plan
-    assert [(s.head_dim, s.window) for s in plan.group_specs] == [(32, 0), (14, 33)] and plan.state_elems == [(2 * 64, "float32")]
+    assert [(s.head_dim, s.window) for s in plan.group_specs] == [(56, 0), (26, 33)] and plan.state_elems == [(2 * 64, "float32")]
 
 
 def test_a_layer_without_a_feed_forward_and_defaults():

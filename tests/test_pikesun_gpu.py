@@ -280,6 +280,22 @@ def test_the_recurrence_carries_its_state_across_portions(name, layer, dtype):
 @pytest.mark.parametrize("name,layer,page", [("P", 0, 8), ("Q", 1, 64), ("Q", 3, 16), ("R", 1, 4), ("R", 2, 32)])
 def test_latent_attention_at_every_edge_of_its_window(name, layer, page, dtype):
     cfg, W = weights_of_layer(name, layer)
+    check_latent_attention(cfg, W, layer, page, dtype)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("heads,dim,rot,vdim,rank,window,page", [(16, 16, 32, 16, 32, 100, 64), (32, 8, 32, 24, 96, 70, 128),
+                                                                 (16, 32, 64, 8, 256, 130, 64), (16, 16, 32, 16, 32, 0, 64)])
+def test_latent_attention_with_heads_in_sixteens(heads, dim, rot, vdim, rank, window, page, dtype):
+    """Sizes that the matrix-core form takes in 16 bits (heads in sixteens, latents in sixteens, key rows
+    in chunks of 32, pages of 64 or 128): its three sizes of register tile."""
+    from pikesun_models import att, config, draw_weights, layer
+    cfg = config(64, 16, [layer(att(heads, dim, rot, vdim, rank, 24, window), None)])
+    W = {k: v for k, v in draw_weights(cfg, 31).items() if k.startswith("l0.")}
+    check_latent_attention(cfg, W, 0, page, dtype, T=330)
+
+
+def check_latent_attention(cfg, W, layer, page, dtype, T=None):
     c = dict(cfg["layers"][layer]["mixer"])
     prefix = f"l{layer}."
     window = c["mask"]["size"] if c.get("mask") else 0
@@ -290,7 +306,7 @@ def test_latent_attention_at_every_edge_of_its_window(name, layer, page, dtype):
         "position": PartSpec("rope", {"head_dim": c["rot_dim"], "rotary_dim": c["rot"]["dims"], "theta": c["rot"]["base"]})})
     c["scale"] *= sharp               # sharp weights: the key that wins decides the row, wherever it lies
     part = build_part("mixer", spec, prefix)
-    T = max(2 * window + 70, 200)
+    T = T or max(2 * window + 70, 200)
     h = rows_in(T, cfg["width"], 13, dtype)
     Wd = {k: v.double() for k, v in W.items()}
     ref = P.latent_attention(Wd, prefix + "mix.", c, h.double(), cfg["norm"]["eps"]).float()
