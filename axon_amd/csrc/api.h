@@ -230,13 +230,17 @@ int axk_grouped_gemm(const void* x, int x_is_f32, long x_row_stride, long x_grou
 // logits (the largest first; of equal ones the lower expert) and the softmax over these.
 // axk_route_sort: the pairs p = t top + k in expert order (sorted, and each one's token in
 // sorted_tokens) and the tiles of the grouped product, at most axk_route_max_tiles of them.
-// axk_route_combine: y[t, :] (+)= sum_k weights[t, k] rows[t top + k, :], k ascending.
+// place_of [n_pairs] (or null): where each pair stands in `sorted`; first_of [n_experts + 1] (or
+// null): where each expert's pairs start there.
+// axk_route_combine: y[t, :] (+)= sum_k weights[t, k] rows[t top + k, :], k ascending (with
+// place_of: rows[place_of[t top + k], :]).  axk_gather_rows: out[r, :] = x[rows[r], :] (elem).
 int axk_route_topk(const float* logits, int n_tokens, int n_experts, int top, int32_t* experts, float* weights, void* stream);
 int axk_route_max_tiles(int n_pairs, int n_experts);
 int axk_route_sort(const int32_t* experts, int n_pairs, int n_experts, int top, int32_t* sorted, int32_t* sorted_tokens,
-                   int32_t* tiles, int32_t* n_tiles, void* stream);
+                   int32_t* tiles, int32_t* n_tiles, int32_t* place_of, int32_t* first_of, void* stream);
 int axk_route_combine(const float* rows, const float* weights, float* y, int n_tokens, int top, int width, int accumulate,
-                      void* stream);
+                      const int32_t* place_of, void* stream);
+int axk_gather_rows(const void* x, long x_stride, const int32_t* rows, void* out, int n_rows, int width, void* stream);
 
 // A short causal convolution per channel and a gated linear recurrence (csrc/recurrent.hip).  A
 // request's state row (float32, rows state_stride apart) holds two copies of ([channels] of
@@ -276,10 +280,13 @@ int axk_latent_prepare(const float* fused, long stride, int q_at, int q_rank, in
                        int table_stride, void* cache, int page_size, void* cq, int n_tokens, int write_kv, void* stream);
 int axk_latent_query_rope(const float* q, int dim, int rot, int rot_dims, const float* table, float* q_full, int rank,
                           int heads, int n_tokens, void* stream);
+// partial: axk_latent_attention_workspace floats (0 for most calls; with few tokens over a window the
+// blocks of 64 positions of a token then run side by side and a second launch folds them), or null.
 int axk_latent_attention_uses_mfma(int heads, int rank, int rot, int page_size);
+long axk_latent_attention_workspace(int n_tokens, int heads, int rank, int rot, int page_size, int window);
 int axk_latent_attention(const float* q_full, const void* cache, const int32_t* block_table, int table_stride,
                          const int32_t* positions, const int32_t* seq_rows, float* o_lat, int n_tokens, int heads, int rank,
-                         int rot, int page_size, int window, float scale, void* stream);
+                         int rot, int page_size, int window, float scale, float* partial, long partial_floats, void* stream);
 
 #ifdef __cplusplus
 }

@@ -168,7 +168,7 @@ __global__ void __launch_bounds__(256)
 latent_attention_mfma_kernel(const float* __restrict__ q_full, const bf16_t* __restrict__ cache,
                              const int32_t* __restrict__ block_table, int table_stride, const int32_t* __restrict__ positions,
                              const int32_t* __restrict__ seq_rows, float* __restrict__ o_lat, int n_tokens, int heads, int rank,
-                             int rot, int page_size, int window, float scale) {
+                             int rot, int page_size, int window, float scale, float* __restrict__ partial, int n_chunks) {
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int groups = heads / 16;
   const long item = (long)blockIdx.x * 4 + wave;
@@ -195,7 +195,11 @@ latent_attention_mfma_kernel(const float* __restrict__ q_full, const bf16_t* __r
 #pragma unroll
   for (int i = 0; i < RT; ++i) acc[i] = la_f32x4{0.0f, 0.0f, 0.0f, 0.0f};
   float m = -INFINITY, l = 0.0f;
-  for (int b = lo / 64; b <= pos / 64; ++b) {
+  // with `partial`: this wave takes one block of 64 positions (blockIdx.y after the token's first) and
+  // leaves (o, m, l) unscaled for the kernel that folds a token's blocks in ascending order
+  const int b_first = partial ? lo / 64 + (int)blockIdx.y : lo / 64;
+  const int b_last = partial ? min(b_first, pos / 64) : pos / 64;
+  for (int b = b_first; b <= b_last; ++b) {
     const int p0 = b * 64, in0 = p0 % page_size;
     const bf16_t* page = cache + (long)pages[p0 / page_size] * page_elems;
     const bf16_t* kbase = page + (long)in0 * width + 8 * g;
@@ -261,6 +265,15 @@ latent_attention_mfma_kernel(const float* __restrict__ q_full, const bf16_t* __r
       }
     }
   }
+  if (partial) {
+    float* dst = partial + (((long)t * heads + hg * 16 + j) * n_chunks + blockIdx.y) * (rank + 2);
+#pragma unroll
+    for (int dt = 0; dt < RT; ++dt)
+      if (dt < rt) *reinterpret_cast<float2*>(dst + 16 * dt + 4 * g) = make_float2(acc[dt][0], acc[dt][1]),
+                   *reinterpret_cast<float2*>(dst + 16 * dt + 4 * g + 2) = make_float2(acc[dt][2], acc[dt][3]);
+    if (g == 0) { dst[rank] = m; dst[rank + 1] = l; }
+    return;
+  }
   const float inv = 1.0f / l;
   float* dst = o_lat + ((long)t * heads + hg * 16 + j) * rank + 4 * g;
 #pragma unroll
@@ -268,14 +281,39 @@ latent_attention_mfma_kernel(const float* __restrict__ q_full, const bf16_t* __r
     if (dt < rt) *reinterpret_cast<float4*>(dst + 16 * dt) = make_float4(acc[dt][0] * inv, acc[dt][1] * inv, acc[dt][2] * inv, acc[dt][3] * inv);
 }
 
+// o_lat[row, :] = sum_c exp(m_c - M) o_c / sum_c exp(m_c - M) l_c over a row's blocks in ascending order
+// (M the largest m_c; a block that saw nothing has l = 0 and is skipped).  One block per (token, head).
+__global__ void latent_attention_fold_kernel(const float* __restrict__ partial, float* __restrict__ o_lat, int rank, int n_chunks) {
+  const float* src = partial + (long)blockIdx.x * n_chunks * (rank + 2);
+  float M = -INFINITY;
+  for (int c = 0; c < n_chunks; ++c)
+    if (src[(long)c * (rank + 2) + rank + 1] > 0.0f) M = fmaxf(M, src[(long)c * (rank + 2) + rank]);
+  float L = 0.0f;
+  for (int c = 0; c < n_chunks; ++c) {
+    const float l = src[(long)c * (rank + 2) + rank + 1];
+    if (l > 0.0f) L = fmaf(expf(src[(long)c * (rank + 2) + rank] - M), l, L);
+  }
+  const float inv = 1.0f / L;
+  for (int d = threadIdx.x; d < rank; d += blockDim.x) {
+    float o = 0.0f;
+    for (int c = 0; c < n_chunks; ++c) {
+      const float l = src[(long)c * (rank + 2) + rank + 1];
+      if (l > 0.0f) o = fmaf(expf(src[(long)c * (rank + 2) + rank] - M), src[(long)c * (rank + 2) + d], o);
+    }
+    o_lat[(long)blockIdx.x * rank + d] = o * inv;
+  }
+}
+
 template <int RT, int QC>
 static void launch_latent_mfma(const float* q_full, const void* cache, const int32_t* block_table, int table_stride,
                                const int32_t* positions, const int32_t* seq_rows, float* o_lat, int n_tokens, int heads, int rank,
-                               int rot, int page_size, int window, float scale, hipStream_t stream) {
+                               int rot, int page_size, int window, float scale, float* partial, int n_chunks, hipStream_t stream) {
   const long items = (long)n_tokens * (heads / 16);
-  latent_attention_mfma_kernel<RT, QC><<<(unsigned)((items + 3) / 4), 256, 0, stream>>>(
+  dim3 grid((unsigned)((items + 3) / 4), partial ? n_chunks : 1);
+  latent_attention_mfma_kernel<RT, QC><<<grid, 256, 0, stream>>>(
       q_full, (const bf16_t*)cache, block_table, table_stride, positions, seq_rows, o_lat, n_tokens, heads, rank, rot, page_size,
-      window, scale);
+      window, scale, partial, n_chunks);
+  if (partial) latent_attention_fold_kernel<<<n_tokens * heads, 128, 0, stream>>>(partial, o_lat, rank, n_chunks);
 }
 #endif
 
@@ -320,9 +358,20 @@ extern "C" int axk_latent_query_rope(const float* q, int dim, int rot, int rot_d
   return 0;
 }
 
+// Few tokens (a decoding step) over a window: a wave per block of 64 positions, so that the blocks of a
+// token run side by side; the floats of the workspace this takes (0: the tokens' waves walk their
+// blocks themselves).  A window of w positions touches at most (w + 62) / 64 + 1 blocks.
+extern "C" long axk_latent_attention_workspace(int n_tokens, int heads, int rank, int rot, int page_size, int window) {
+  if (!axk_latent_attention_uses_mfma(heads, rank, rot, page_size) || window <= 0) return 0;
+  const int blocks = (window + 62) / 64 + 1;
+  if (blocks < 2 || (long)n_tokens * (heads / 16) >= 512) return 0;
+  return (long)n_tokens * heads * blocks * (rank + 2);
+}
+
 extern "C" int axk_latent_attention(const float* q_full, const void* cache, const int32_t* block_table, int table_stride,
                                     const int32_t* positions, const int32_t* seq_rows, float* o_lat, int n_tokens, int heads,
-                                    int rank, int rot, int page_size, int window, float scale, void* stream) {
+                                    int rank, int rot, int page_size, int window, float scale, float* partial,
+                                    long partial_floats, void* stream) {
   AXK_REQUIRE(n_tokens >= 0 && heads > 0 && rank > 0 && rot >= 0 && page_size > 0 && window >= 0,
               "latent_attention: bad sizes T=%d heads=%d rank=%d rot=%d page=%d window=%d", n_tokens, heads, rank, rot,
               page_size, window);
@@ -333,15 +382,20 @@ extern "C" int axk_latent_attention(const float* q_full, const void* cache, cons
   if (axk_latent_attention_uses_mfma(heads, rank, rot, page_size) && ((uintptr_t)q_full & 15) == 0 && ((uintptr_t)cache & 15) == 0 &&
       ((uintptr_t)o_lat & 15) == 0) {
     hipStream_t s = (hipStream_t)stream;
+    const long need = axk_latent_attention_workspace(n_tokens, heads, rank, rot, page_size, window);
+    AXK_REQUIRE(partial == nullptr || partial_floats >= need, "latent_attention: a workspace of %ld floats, %ld needed",
+                partial_floats, need);
+    if (need == 0) partial = nullptr;
+    const int n_chunks = (window + 62) / 64 + 1;
     if (rank <= 64 && rank + rot <= 128)
       launch_latent_mfma<4, 4>(q_full, cache, block_table, table_stride, positions, seq_rows, o_lat, n_tokens, heads, rank, rot,
-                               page_size, window, scale, s);
+                               page_size, window, scale, partial, n_chunks, s);
     else if (rank <= 128 && rank + rot <= 256)
       launch_latent_mfma<8, 8>(q_full, cache, block_table, table_stride, positions, seq_rows, o_lat, n_tokens, heads, rank, rot,
-                               page_size, window, scale, s);
+                               page_size, window, scale, partial, n_chunks, s);
     else
       launch_latent_mfma<32, 20>(q_full, cache, block_table, table_stride, positions, seq_rows, o_lat, n_tokens, heads, rank, rot,
-                                 page_size, window, scale, s);
+                                 page_size, window, scale, partial, n_chunks, s);
     AXK_LAUNCH_CHECK("latent_attention");
     return 0;
   }

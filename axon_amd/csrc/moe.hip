@@ -42,7 +42,8 @@ __global__ void route_topk_kernel(const float* __restrict__ logits, int n_tokens
 // depends on it: every row of a product is a chain of its own.
 __global__ void __launch_bounds__(1024)
 route_sort_kernel(const int32_t* __restrict__ experts, int n_pairs, int n_experts, int top, int32_t* __restrict__ sorted,
-                  int32_t* __restrict__ sorted_tokens, int32_t* __restrict__ tiles, int32_t* __restrict__ n_tiles) {
+                  int32_t* __restrict__ sorted_tokens, int32_t* __restrict__ tiles, int32_t* __restrict__ n_tiles,
+                  int32_t* __restrict__ place_of, int32_t* __restrict__ first_of) {
   extern __shared__ int counts[];              // [n_experts] counts, then [n_experts] next free places
   int* next = counts + n_experts;
   for (int e = threadIdx.x; e < n_experts; e += blockDim.x) counts[e] = 0;
@@ -54,6 +55,7 @@ route_sort_kernel(const int32_t* __restrict__ experts, int n_pairs, int n_expert
     for (int e = 0; e < n_experts; ++e) {
       const int n = counts[e];
       next[e] = at;
+      if (first_of) first_of[e] = at;
       for (int i = 0; i < n; i += 16) {
         tiles[3 * tile] = e; tiles[3 * tile + 1] = at + i; tiles[3 * tile + 2] = min(16, n - i);
         ++tile;
@@ -61,24 +63,38 @@ route_sort_kernel(const int32_t* __restrict__ experts, int n_pairs, int n_expert
       at += n;
     }
     *n_tiles = tile;
+    if (first_of) first_of[n_experts] = at;
   }
   __syncthreads();
   for (int p = threadIdx.x; p < n_pairs; p += blockDim.x) {
     const int place = atomicAdd(&next[experts[p]], 1);
     sorted[place] = p;
     sorted_tokens[place] = p / top;
+    if (place_of) place_of[p] = place;
   }
 }
 
-// y[t, :] (+)= sum_k weights[t, k] rows[t top + k, :], k ascending.
+// y[t, :] (+)= sum_k weights[t, k] rows[row of pair t top + k, :], k ascending; a pair's row is the pair
+// itself, or place_of[pair].
 __global__ void route_combine_kernel(const float* __restrict__ rows, const float* __restrict__ weights, float* __restrict__ y,
-                                     int top, int width, int accumulate) {
+                                     int top, int width, int accumulate, const int32_t* __restrict__ place_of) {
   const int t = blockIdx.y;
   const int c = blockIdx.x * blockDim.x + threadIdx.x;
   if (c >= width) return;
   float acc = accumulate ? y[(long)t * width + c] : 0.0f;
-  for (int k = 0; k < top; ++k) acc = fmaf(weights[(long)t * top + k], rows[((long)t * top + k) * width + c], acc);
+  for (int k = 0; k < top; ++k) {
+    const long pair = (long)t * top + k;
+    acc = fmaf(weights[pair], rows[(place_of ? (long)place_of[pair] : pair) * width + c], acc);
+  }
   y[(long)t * width + c] = acc;
+}
+
+// out[r, :] = x[rows[r], :] (rows of the compute dtype).
+__global__ void gather_rows_kernel(const elem_t* __restrict__ x, long x_stride, const int32_t* __restrict__ rows,
+                                   elem_t* __restrict__ out, int width) {
+  const elem_t* src = x + (long)rows[blockIdx.x] * x_stride;
+  elem_t* dst = out + (long)blockIdx.x * width;
+  for (int i = threadIdx.x; i < width; i += blockDim.x) dst[i] = src[i];
 }
 
 }  // namespace
@@ -95,23 +111,32 @@ extern "C" int axk_route_topk(const float* logits, int n_tokens, int n_experts, 
 
 extern "C" int axk_route_max_tiles(int n_pairs, int n_experts) { return ceil_div(n_pairs, 16) + n_experts; }
 
+extern "C" int axk_gather_rows(const void* x, long x_stride, const int32_t* rows, void* out, int n_rows, int width, void* stream) {
+  AXK_REQUIRE(n_rows >= 0 && width > 0 && x_stride >= width, "gather_rows: %d rows of %d (stride %ld)", n_rows, width, x_stride);
+  if (n_rows == 0) return 0;
+  gather_rows_kernel<<<n_rows, 256, 0, (hipStream_t)stream>>>((const elem_t*)x, x_stride, rows, (elem_t*)out, width);
+  AXK_LAUNCH_CHECK("gather_rows");
+  return 0;
+}
+
 extern "C" int axk_route_sort(const int32_t* experts, int n_pairs, int n_experts, int top, int32_t* sorted,
-                              int32_t* sorted_tokens, int32_t* tiles, int32_t* n_tiles, void* stream) {
+                              int32_t* sorted_tokens, int32_t* tiles, int32_t* n_tiles, int32_t* place_of, int32_t* first_of,
+                              void* stream) {
   AXK_REQUIRE(n_pairs >= 0 && n_experts > 0 && top > 0 && n_experts <= 4096, "route_sort: %d pairs, %d experts", n_pairs,
               n_experts);
   route_sort_kernel<<<1, 1024, 2 * n_experts * sizeof(int), (hipStream_t)stream>>>(experts, n_pairs, n_experts, top, sorted,
-                                                                                  sorted_tokens, tiles, n_tiles);
+                                                                                  sorted_tokens, tiles, n_tiles, place_of, first_of);
   AXK_LAUNCH_CHECK("route_sort");
   return 0;
 }
 
 extern "C" int axk_route_combine(const float* rows, const float* weights, float* y, int n_tokens, int top, int width,
-                                 int accumulate, void* stream) {
+                                 int accumulate, const int32_t* place_of, void* stream) {
   AXK_REQUIRE(n_tokens >= 0 && top > 0 && width > 0 && n_tokens <= 65535, "route_combine: T=%d top=%d width=%d", n_tokens, top,
               width);
   if (n_tokens == 0) return 0;
   dim3 grid(ceil_div(width, 256), n_tokens);
-  route_combine_kernel<<<grid, 256, 0, (hipStream_t)stream>>>(rows, weights, y, top, width, accumulate);
+  route_combine_kernel<<<grid, 256, 0, (hipStream_t)stream>>>(rows, weights, y, top, width, accumulate, place_of);
   AXK_LAUNCH_CHECK("route_combine");
   return 0;
 }

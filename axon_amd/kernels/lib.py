@@ -84,8 +84,9 @@ _SIGNATURES = {
                          c_int, c_void_p],
     "axk_route_topk": [c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p],
     "axk_route_max_tiles": [c_int, c_int],
-    "axk_route_sort": [c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p],
-    "axk_route_combine": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
+    "axk_route_sort": [c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p],
+    "axk_route_combine": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p, c_void_p],
+    "axk_gather_rows": [c_void_p, c_long, c_void_p, c_void_p, c_int, c_int, c_void_p],
     "axk_causal_conv": [c_void_p, c_long, c_void_p, c_void_p, c_int, c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_int, c_int,
                         c_int, c_void_p],
     "axk_gated_scan": [c_void_p, c_void_p, c_void_p, c_long, c_void_p, c_long, c_void_p, c_int, c_float, c_void_p, c_long,
@@ -94,7 +95,7 @@ _SIGNATURES = {
                            c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_int, c_void_p],
     "axk_latent_query_rope": [c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],
     "axk_latent_attention": [c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
-                             c_int, c_int, c_float, c_void_p],
+                             c_int, c_int, c_float, c_void_p, c_long, c_void_p],
     "axk_fill_i32": [c_void_p, c_int, c_int, c_void_p],
     "axk_fill_f32": [c_void_p, c_float, c_int, c_void_p],
 }
@@ -144,6 +145,8 @@ class Kernels:
             fn.restype = c_int
         self.lib.axk_attention_decode_workspace.argtypes = [c_int, c_int, c_int, c_int]
         self.lib.axk_attention_decode_workspace.restype = ctypes.c_long
+        self.lib.axk_latent_attention_workspace.argtypes = [c_int, c_int, c_int, c_int, c_int, c_int]
+        self.lib.axk_latent_attention_workspace.restype = ctypes.c_long
         self.lib.axk_packed_elems.argtypes = [c_int, c_int]
         self.lib.axk_packed_elems.restype = ctypes.c_long
         self.lib.axk_gemm_workspace.argtypes = [c_int, c_int, c_int, c_int]
@@ -204,7 +207,7 @@ class Kernels:
     _LAUNCHING = ("embed", "rmsnorm", "rope_table", "rope_kv_write", "gemm_qkv_rope", "attention", "attention_prefill",
                   "attention_decode", "gemm", "gemm_normed_glu", "gemm_normed_qkv_rope", "swiglu", "argmax", "topk",
                   "fill_i32", "fill_f32", "call", "norm_add", "round_rows", "activation", "clamped_glu", "grouped_gemm",
-                  "route_topk", "route_sort", "route_combine", "causal_conv", "gated_scan", "latent_prepare",
+                  "route_topk", "route_sort", "route_combine", "gather_rows", "causal_conv", "gated_scan", "latent_prepare",
                   "latent_query_rope", "latent_attention")
     _MATRIX_AT = {"gemm": 1, "gemm_qkv_rope": 1, "gemm_normed_glu": 3, "gemm_normed_qkv_rope": 3, "grouped_gemm": 1}   # which argument is W
 
@@ -736,22 +739,37 @@ class Kernels:
     def route_max_tiles(self, n_pairs: int, n_experts: int) -> int:
         return int(self.lib.axk_route_max_tiles(n_pairs, n_experts))
 
-    def route_sort(self, experts: torch.Tensor, n_experts: int, sorted_pairs, sorted_tokens, tiles, n_tiles) -> None:
-        for t in (experts, sorted_pairs, sorted_tokens, tiles, n_tiles):
+    def route_sort(self, experts: torch.Tensor, n_experts: int, sorted_pairs, sorted_tokens, tiles, n_tiles, place_of=None,
+                   first_of=None) -> None:
+        """The pairs in expert order, their tokens, the grouped product's tiles; optionally where each
+        pair stands (place_of [pairs]) and where each expert's pairs start (first_of [experts + 1])."""
+        for t in (experts, sorted_pairs, sorted_tokens, tiles, n_tiles) + tuple(t for t in (place_of, first_of) if t is not None):
             self._i32(t, "route_sort")
+        if (place_of is not None and place_of.numel() < experts.numel()) or (first_of is not None and first_of.numel() < n_experts + 1):
+            raise KernelError("route_sort: place_of or first_of is too short")
         P = experts.numel()
         if sorted_pairs.numel() < P or sorted_tokens.numel() < P or tiles.numel() < 3 * self.route_max_tiles(P, n_experts):
             raise KernelError(f"route_sort: lists too short for {P} pairs of {n_experts} experts")
         self._check(self.lib.axk_route_sort(_ptr(experts), P, n_experts, experts.shape[-1], _ptr(sorted_pairs), _ptr(sorted_tokens),
-                                            _ptr(tiles), _ptr(n_tiles), _stream()))
+                                            _ptr(tiles), _ptr(n_tiles), _ptr(place_of), _ptr(first_of), _stream()))
 
-    def route_combine(self, rows: torch.Tensor, weights: torch.Tensor, y: torch.Tensor, accumulate: bool = False) -> torch.Tensor:
+    def gather_rows(self, x: torch.Tensor, rows: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+        self._elem(x, "gather x"); self._elem(out, "gather out"); self._i32(rows, "gather rows")
+        if out.shape != (rows.numel(), x.shape[1]) or x.stride(1) != 1 or not out.is_contiguous():
+            raise KernelError(f"gather_rows: {rows.numel()} rows of {tuple(x.shape)} into {tuple(out.shape)}")
+        self._check(self.lib.axk_gather_rows(_ptr(x), x.stride(0), _ptr(rows), _ptr(out), rows.numel(), x.shape[1], _stream()))
+        return out
+
+    def route_combine(self, rows: torch.Tensor, weights: torch.Tensor, y: torch.Tensor, accumulate: bool = False,
+                      place_of: Optional[torch.Tensor] = None) -> torch.Tensor:
         self._f32(rows, "expert rows"); self._f32(weights, "router weights"); self._f32(y, "combine y")
+        if place_of is not None:
+            self._i32(place_of, "combine place_of")
         T, top = weights.shape
         if rows.shape != (T * top, y.shape[1]) or y.shape[0] != T:
             raise KernelError(f"route_combine: rows {tuple(rows.shape)}, weights {tuple(weights.shape)}, y {tuple(y.shape)}")
         self._check(self.lib.axk_route_combine(_ptr(rows), _ptr(weights), _ptr(y), T, top, y.shape[1], 1 if accumulate else 0,
-                                               _stream()))
+                                               _ptr(place_of), _stream()))
         return y
 
     # ------------------------------------------------------------------ convolution and recurrence with per-request state
@@ -836,9 +854,11 @@ class Kernels:
             raise KernelError(f"latent_attention: q_full {tuple(q_full.shape)}, o_lat {tuple(o_lat.shape)} for {T} tokens")
         if cache.dim() != 4 or tuple(cache.shape[1:]) != (1, page_size, 2 * rank + rot) or not cache.is_contiguous():
             raise KernelError(f"latent_attention: cache {tuple(cache.shape)} is not [pages, 1, {page_size}, {2 * rank + rot}]")
+        need = int(self.lib.axk_latent_attention_workspace(T, heads, rank, rot, page_size, int(window)))
+        partial = torch.empty(need, dtype=torch.float32, device=o_lat.device) if need else None
         self._check(self.lib.axk_latent_attention(_ptr(q_full), _ptr(cache), _ptr(block_table), block_table.shape[-1],
                                                   _ptr(positions), _ptr(seq_rows), _ptr(o_lat), T, heads, rank, rot, page_size,
-                                                  int(window), float(scale), _stream()))
+                                                  int(window), float(scale), _ptr(partial), need, _stream()))
         return o_lat
 
     def fill_i32(self, dst: torch.Tensor, value: int) -> None:

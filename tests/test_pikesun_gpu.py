@@ -292,7 +292,8 @@ def test_latent_attention_with_heads_in_sixteens(heads, dim, rot, vdim, rank, wi
     from pikesun_models import att, config, draw_weights, layer
     cfg = config(64, 16, [layer(att(heads, dim, rot, vdim, rank, 24, window), None)])
     W = {k: v for k, v in draw_weights(cfg, 31).items() if k.startswith("l0.")}
-    check_latent_attention(cfg, W, 0, page, dtype, T=330)
+    # few tokens over a window: a token's blocks of positions side by side and folded; many tokens: a wave walks them
+    check_latent_attention(cfg, W, 0, page, dtype, T=600 if heads == 32 else 330)
 
 
 def check_latent_attention(cfg, W, layer, page, dtype, T=None):
@@ -312,7 +313,7 @@ def check_latent_attention(cfg, W, layer, page, dtype, T=None):
     ref = P.latent_attention(Wd, prefix + "mix.", c, h.double(), cfg["norm"]["eps"]).float()
     first = max(window - 3, 2)
     for cuts in ([T], [first] + [1] * 8 + [T - first - 8], [2, 1, 1, 3] + [1] * 30 + [64, 2, T - 103]):
-        hs = PartHarness(dtype, part.cache_spec(), page_size=page, n_pages=-(-T // page) + 3, max_seq_len=512)
+        hs = PartHarness(dtype, part.cache_spec(), page_size=page, n_pages=-(-T // page) + 3, max_seq_len=1024)
         part.load(WeightStore(DictSource(W), hs.rt.device, hs.rt.dtype), hs.rt)
         got = run_mixer(part, hs, h, cuts, cfg["width"])
         assert float((got - ref).abs().max()) <= part_tol(dtype, ref), cuts
@@ -366,17 +367,21 @@ def test_feed_forwards_alone(name, layer, dtype):
     prefix = f"l{layer}."
     spec = config_from_dict(cfg).layers[layer]["mlp"]
     part = build_part("feed_forward", spec, prefix)
-    hs = PartHarness(dtype, CacheSpec(entries=1, heads=1, head_dim=8))
+    hs = PartHarness(dtype, CacheSpec(entries=1, heads=1, head_dim=8), page_size=64, n_pages=16, max_seq_len=1024)
     part.load(WeightStore(DictSource(W), hs.rt.device, hs.rt.dtype), hs.rt)
     Wd = {k: v.double() for k, v in W.items()}
-    for T in (1, 5, 70):
+    for T in (1, 5, 70, 400):            # 400 rows: experts with many rows each run one by one through the large products
         h = rows_in(T, cfg["width"], 19 + T, dtype) * 1.5
         ref = P.feed_forward(Wd, prefix + "mlp.", mlp, h.double()).float()
         ctx = hs.ctx([0] * T)
         out = torch.full((T, cfg["width"]), float("nan"), dtype=torch.float32, device="cuda")
         part.forward(ctx, h.to(hs.rt.dtype).cuda(), out, accumulate=False)
         err = (out.cpu() - ref).abs().max(dim=-1).values
-        # in 16 bits the router's operand is rounded as in the plain run (the rows are bfloat16 values): no close calls
+        if mlp["kind"] == "moe" and mlp["router"]["top"] < mlp["router"]["experts"]:
+            # a row whose last chosen expert and first left out are a close call may go either way: not this test's matter
+            z = (h.double() @ Wd[prefix + "mlp.router"].T).sort(dim=-1, descending=True).values
+            top = mlp["router"]["top"]
+            err = err[(z[:, top - 1] - z[:, top]) > 0.05]
         assert float(err.max()) <= part_tol(dtype, ref), (T, int(err.argmax()))
         again = torch.ones((T, cfg["width"]), dtype=torch.float32, device="cuda")
         part.forward(ctx, h.to(hs.rt.dtype).cuda(), again)               # added into rows that hold something
