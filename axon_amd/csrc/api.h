@@ -213,7 +213,8 @@ int axk_clamped_glu(const void* gate_up, void* out, int n_tokens, int n_ffn, flo
 //   out[orow(r), g ogs + n] = epilogue(sum_k X[xrow(r), g xgs + k] W[g][n][k] + bias[g][n]),
 // W elem [groups][n (2 n with glu)][k].  tiles == null: every row r < m meets every group
 // (block-diagonal; x_rows and out_rows must be null).  tiles [.][3] = (group, first listed row,
-// count <= 16) with *n_tiles of them on the device (max_tiles: the most there can be): the rows
+// count <= tile_rows) with *n_tiles of them on the device (max_tiles: the most there can be;
+// tile_rows 16, or 64 for many rows a group: tiles through LDS, the same chains, the same bits): the rows
 // listed, x_rows / out_rows naming the row of X each reads and the row of out it writes (null:
 // the listed row itself).  glu: g = min(gate, limit), u = clamp(up, -limit, limit), out = g
 // sigmoid(alpha g) (u + 1).  gate (float32, rows gate_row_stride apart): out is multiplied by
@@ -223,21 +224,22 @@ int axk_grouped_gemm_uses_mfma(int k, int x_is_f32, long x_row_stride, long x_gr
 int axk_grouped_gemm(const void* x, int x_is_f32, long x_row_stride, long x_group_stride, const int32_t* x_rows,
                      const void* w, const void* bias, int bias_is_f32, void* out, int out_is_f32, long out_row_stride,
                      long out_group_stride, const int32_t* out_rows, const float* gate, long gate_row_stride, int glu,
-                     float glu_limit, float glu_alpha, const int32_t* tiles, const int32_t* n_tiles, int max_tiles, int m,
-                     int n, int k, int groups, void* stream);
+                     float glu_limit, float glu_alpha, const int32_t* tiles, const int32_t* n_tiles, int max_tiles,
+                     int tile_rows, int m, int n, int k, int groups, void* stream);
 
 // Routing (csrc/moe.hip).  axk_route_topk: for each token the `top` largest of its n_experts
 // logits (the largest first; of equal ones the lower expert) and the softmax over these.
 // axk_route_sort: the pairs p = t top + k in expert order (sorted, and each one's token in
-// sorted_tokens) and the tiles of the grouped product, at most axk_route_max_tiles of them.
+// sorted_tokens) and the tiles (of up to tile_rows rows) of the grouped product, at most
+// axk_route_max_tiles of them.
 // place_of [n_pairs] (or null): where each pair stands in `sorted`; first_of [n_experts + 1] (or
 // null): where each expert's pairs start there.
 // axk_route_combine: y[t, :] (+)= sum_k weights[t, k] rows[t top + k, :], k ascending (with
 // place_of: rows[place_of[t top + k], :]).  axk_gather_rows: out[r, :] = x[rows[r], :] (elem).
 int axk_route_topk(const float* logits, int n_tokens, int n_experts, int top, int32_t* experts, float* weights, void* stream);
-int axk_route_max_tiles(int n_pairs, int n_experts);
+int axk_route_max_tiles(int n_pairs, int n_experts, int tile_rows);
 int axk_route_sort(const int32_t* experts, int n_pairs, int n_experts, int top, int32_t* sorted, int32_t* sorted_tokens,
-                   int32_t* tiles, int32_t* n_tiles, int32_t* place_of, int32_t* first_of, void* stream);
+                   int32_t* tiles, int32_t* n_tiles, int32_t* place_of, int32_t* first_of, int tile_rows, void* stream);
 int axk_route_combine(const float* rows, const float* weights, float* y, int n_tokens, int top, int width, int accumulate,
                       const int32_t* place_of, void* stream);
 int axk_gather_rows(const void* x, long x_stride, const int32_t* rows, void* out, int n_rows, int width, void* stream);

@@ -26,7 +26,7 @@ enum {
   INST_ATTENTION_PREFILL,    // head_dim, query heads a block, pages of 64 positions or more
   INST_ATTENTION_DECODE,     // head_dim, waves a block
   INST_RMSNORM,              // 1: rows read as float4
-  INST_GROUPED_GEMM,         // 1: matrix cores, 0: 32-bit FMA; gated epilogue
+  INST_GROUPED_GEMM,         // 2: matrix cores through LDS, 1: matrix cores from memory, 0: 32-bit FMA; gated epilogue
   INST_KINDS
 };
 

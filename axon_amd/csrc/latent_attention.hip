@@ -154,7 +154,7 @@ typedef __attribute__((ext_vector_type(8))) __bf16 la_bf16x8;
 typedef __attribute__((ext_vector_type(4))) float la_f32x4;
 __device__ inline la_bf16x8 la_frag(uint4 v) { return __builtin_bit_cast(la_bf16x8, v); }
 
-// The same attention on the matrix cores.  One wave per (token, sixteen heads), four waves a block,
+// The same attention on the matrix cores.  One wave per (token, sixteen heads), two waves a block,
 // each on its own: the sixteen heads of a token see the same positions, so a block of 64 positions is
 //   S^T [position, head] = K [position, dims] Q^T           (rank + rot dims in chunks of 32),
 //   a maximum, weights and their sum per head (a lane holds 16 positions of its head; the four
@@ -163,30 +163,38 @@ __device__ inline la_bf16x8 la_frag(uint4 v) { return __builtin_bit_cast(la_bf16
 // with K rows and the rows of C^T straight from the page into the first operand (16 or 8 bytes a
 // lane) and the rounded weights, as they lie in the accumulators, as the second.  RT: tiles of 16
 // latent dims at most; QC: chunks of 32 key dims at most.  Pages hold a multiple of 64 positions.
+#define LAM_WAVES 2
 template <int RT, int QC>
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(LAM_WAVES * 64)
 latent_attention_mfma_kernel(const float* __restrict__ q_full, const bf16_t* __restrict__ cache,
                              const int32_t* __restrict__ block_table, int table_stride, const int32_t* __restrict__ positions,
                              const int32_t* __restrict__ seq_rows, float* __restrict__ o_lat, int n_tokens, int heads, int rank,
                              int rot, int page_size, int window, float scale, float* __restrict__ partial, int n_chunks) {
+  // the sixteen heads' queries as bfloat16 in LDS, rows 16 bytes longer than their chunks so that the
+  // sixteen rows a product's operand is read from fall into different banks
+  constexpr int QROW = QC * 32 + 8;
+  __shared__ __align__(16) bf16_t qs_all[LAM_WAVES][16 * QROW];
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int groups = heads / 16;
-  const long item = (long)blockIdx.x * 4 + wave;
-  if (item >= (long)n_tokens * groups) return;
-  const int t = (int)(item / groups), hg = (int)(item % groups);
+  const long item = (long)blockIdx.x * LAM_WAVES + wave;
+  const bool active = item < (long)n_tokens * groups;
+  const int t = active ? (int)(item / groups) : 0, hg = active ? (int)(item % groups) : 0;
   const int width = rank + rot, qc = width / 32, rt = rank / 16;
   const int j = lane & 15, g = lane >> 4;
-  const float* qrow = q_full + ((long)t * heads + hg * 16 + j) * width + 8 * g;
-  uint4 qf[QC];
-#pragma unroll
-  for (int kc = 0; kc < QC; ++kc) {
-    if (kc < qc) {
-      const float4 a = *reinterpret_cast<const float4*>(qrow + 32 * kc), b = *reinterpret_cast<const float4*>(qrow + 32 * kc + 4);
-      qf[kc] = make_uint4(pack2_bf16(a.x, a.y), pack2_bf16(a.z, a.w), pack2_bf16(b.x, b.y), pack2_bf16(b.z, b.w));
-    } else {
-      qf[kc] = make_uint4(0, 0, 0, 0);
+  bf16_t* qs = qs_all[wave];
+  if (active) {
+    const int per_row = width / 8;
+    for (int idx = lane; idx < 16 * per_row; idx += 64) {
+      const int row = idx / per_row, part = idx % per_row;
+      const float* src = q_full + ((long)t * heads + hg * 16 + row) * width + 8 * part;
+      const float4 a = *reinterpret_cast<const float4*>(src), b = *reinterpret_cast<const float4*>(src + 4);
+      *reinterpret_cast<uint4*>(qs + row * QROW + 8 * part) =
+          make_uint4(pack2_bf16(a.x, a.y), pack2_bf16(a.z, a.w), pack2_bf16(b.x, b.y), pack2_bf16(b.z, b.w));
     }
   }
+  __syncthreads();
+  if (!active) return;
+  const bf16_t* qlane = qs + j * QROW + 8 * g;
   const int pos = positions[t];
   const int lo = window > 0 ? max(0, pos + 1 - window) : 0;
   const int32_t* pages = block_table + (long)seq_rows[t] * table_stride;
@@ -209,11 +217,17 @@ latent_attention_mfma_kernel(const float* __restrict__ q_full, const bf16_t* __r
     for (int pt = 0; pt < 4; ++pt) {
       s[pt] = la_f32x4{0.0f, 0.0f, 0.0f, 0.0f};
       const bf16_t* krow = kbase + (long)(16 * pt + j) * width;
+      constexpr int QB = QC < 10 ? QC : 10;         // chunks of a row asked for before the first product waits for any
 #pragma unroll
-      for (int kc = 0; kc < QC; ++kc)
-        if (kc < qc)
-          s[pt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(la_frag(*reinterpret_cast<const uint4*>(krow + 32 * kc)),
-                                                          la_frag(qf[kc]), s[pt], 0, 0, 0);
+      for (int k0 = 0; k0 < QC; k0 += QB) {
+        uint4 kf[QB];
+#pragma unroll
+        for (int e = 0; e < QB; ++e)
+          if (k0 + e < qc) kf[e] = *reinterpret_cast<const uint4*>(krow + 32 * (k0 + e));
+#pragma unroll
+        for (int e = 0; e < QB; ++e)
+          if (k0 + e < qc) s[pt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(la_frag(kf[e]), la_frag(*reinterpret_cast<const uint4*>(qlane + 32 * (k0 + e))), s[pt], 0, 0, 0);
+      }
     }
     float mx = -INFINITY;
 #pragma unroll
@@ -247,21 +261,31 @@ latent_attention_mfma_kernel(const float* __restrict__ q_full, const bf16_t* __r
     for (int c = 0; c < 2; ++c)
       pf[c] = make_uint4(pack2_bf16(s[2 * c][0], s[2 * c][1]), pack2_bf16(s[2 * c][2], s[2 * c][3]),
                          pack2_bf16(s[2 * c + 1][0], s[2 * c + 1][1]), pack2_bf16(s[2 * c + 1][2], s[2 * c + 1][3]));
+    constexpr int VB = 4;                         // tiles of 16 dims whose rows are asked for together
 #pragma unroll
-    for (int dt = 0; dt < RT; ++dt) {
-      if (dt < rt) {
-        const bf16_t* vrow = vbase + (long)(16 * dt + j) * page_size;
-        uint2 v[4];
+    for (int d0 = 0; d0 < RT; d0 += VB) {
+      uint2 v[VB][4];
 #pragma unroll
-        for (int c = 0; c < 2; ++c) {
-          v[2 * c] = *reinterpret_cast<const uint2*>(vrow + 32 * c);
-          v[2 * c + 1] = *reinterpret_cast<const uint2*>(vrow + 32 * c + 16);
+      for (int e = 0; e < VB; ++e) {
+        if (d0 + e < rt) {
+          const bf16_t* vrow = vbase + (long)(16 * (d0 + e) + j) * page_size;
+#pragma unroll
+          for (int c = 0; c < 2; ++c) {
+            v[e][2 * c] = *reinterpret_cast<const uint2*>(vrow + 32 * c);
+            v[e][2 * c + 1] = *reinterpret_cast<const uint2*>(vrow + 32 * c + 16);
+          }
         }
-        acc[dt] *= fold;
+      }
 #pragma unroll
-        for (int c = 0; c < 2; ++c)
-          acc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(la_frag(make_uint4(v[2 * c].x, v[2 * c].y, v[2 * c + 1].x, v[2 * c + 1].y)),
-                                                            la_frag(pf[c]), acc[dt], 0, 0, 0);
+      for (int e = 0; e < VB; ++e) {
+        if (d0 + e < rt) {
+          acc[d0 + e] *= fold;
+#pragma unroll
+          for (int c = 0; c < 2; ++c)
+            acc[d0 + e] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                la_frag(make_uint4(v[e][2 * c].x, v[e][2 * c].y, v[e][2 * c + 1].x, v[e][2 * c + 1].y)), la_frag(pf[c]), acc[d0 + e],
+                0, 0, 0);
+        }
       }
     }
   }
@@ -309,8 +333,8 @@ static void launch_latent_mfma(const float* q_full, const void* cache, const int
                                const int32_t* positions, const int32_t* seq_rows, float* o_lat, int n_tokens, int heads, int rank,
                                int rot, int page_size, int window, float scale, float* partial, int n_chunks, hipStream_t stream) {
   const long items = (long)n_tokens * (heads / 16);
-  dim3 grid((unsigned)((items + 3) / 4), partial ? n_chunks : 1);
-  latent_attention_mfma_kernel<RT, QC><<<grid, 256, 0, stream>>>(
+  dim3 grid((unsigned)((items + LAM_WAVES - 1) / LAM_WAVES), partial ? n_chunks : 1);
+  latent_attention_mfma_kernel<RT, QC><<<grid, LAM_WAVES * 64, 0, stream>>>(
       q_full, (const bf16_t*)cache, block_table, table_stride, positions, seq_rows, o_lat, n_tokens, heads, rank, rot, page_size,
       window, scale, partial, n_chunks);
   if (partial) latent_attention_fold_kernel<<<n_tokens * heads, 128, 0, stream>>>(partial, o_lat, rank, n_chunks);

@@ -37,13 +37,13 @@ __global__ void route_topk_kernel(const float* __restrict__ logits, int n_tokens
 }
 
 // One block.  pairs p = t top + k in expert order -> sorted [n_pairs], with the token of each
-// (sorted_tokens); tiles [.][3] = (expert, first place in sorted, count <= 16), *n_tiles of them.
+// (sorted_tokens); tiles [.][3] = (expert, first place in sorted, count <= tile_rows), *n_tiles of them.
 // Which place a pair gets inside its expert's stretch is not fixed (atomic counters); no result
 // depends on it: every row of a product is a chain of its own.
 __global__ void __launch_bounds__(1024)
 route_sort_kernel(const int32_t* __restrict__ experts, int n_pairs, int n_experts, int top, int32_t* __restrict__ sorted,
                   int32_t* __restrict__ sorted_tokens, int32_t* __restrict__ tiles, int32_t* __restrict__ n_tiles,
-                  int32_t* __restrict__ place_of, int32_t* __restrict__ first_of) {
+                  int32_t* __restrict__ place_of, int32_t* __restrict__ first_of, int tile_rows) {
   extern __shared__ int counts[];              // [n_experts] counts, then [n_experts] next free places
   int* next = counts + n_experts;
   for (int e = threadIdx.x; e < n_experts; e += blockDim.x) counts[e] = 0;
@@ -56,8 +56,8 @@ route_sort_kernel(const int32_t* __restrict__ experts, int n_pairs, int n_expert
       const int n = counts[e];
       next[e] = at;
       if (first_of) first_of[e] = at;
-      for (int i = 0; i < n; i += 16) {
-        tiles[3 * tile] = e; tiles[3 * tile + 1] = at + i; tiles[3 * tile + 2] = min(16, n - i);
+      for (int i = 0; i < n; i += tile_rows) {
+        tiles[3 * tile] = e; tiles[3 * tile + 1] = at + i; tiles[3 * tile + 2] = min(tile_rows, n - i);
         ++tile;
       }
       at += n;
@@ -109,7 +109,9 @@ extern "C" int axk_route_topk(const float* logits, int n_tokens, int n_experts, 
   return 0;
 }
 
-extern "C" int axk_route_max_tiles(int n_pairs, int n_experts) { return ceil_div(n_pairs, 16) + n_experts; }
+extern "C" int axk_route_max_tiles(int n_pairs, int n_experts, int tile_rows) {
+  return ceil_div(n_pairs, tile_rows > 0 ? tile_rows : 16) + n_experts;
+}
 
 extern "C" int axk_gather_rows(const void* x, long x_stride, const int32_t* rows, void* out, int n_rows, int width, void* stream) {
   AXK_REQUIRE(n_rows >= 0 && width > 0 && x_stride >= width, "gather_rows: %d rows of %d (stride %ld)", n_rows, width, x_stride);
@@ -121,11 +123,11 @@ extern "C" int axk_gather_rows(const void* x, long x_stride, const int32_t* rows
 
 extern "C" int axk_route_sort(const int32_t* experts, int n_pairs, int n_experts, int top, int32_t* sorted,
                               int32_t* sorted_tokens, int32_t* tiles, int32_t* n_tiles, int32_t* place_of, int32_t* first_of,
-                              void* stream) {
-  AXK_REQUIRE(n_pairs >= 0 && n_experts > 0 && top > 0 && n_experts <= 4096, "route_sort: %d pairs, %d experts", n_pairs,
-              n_experts);
+                              int tile_rows, void* stream) {
+  AXK_REQUIRE(n_pairs >= 0 && n_experts > 0 && top > 0 && n_experts <= 4096 && tile_rows > 0,
+              "route_sort: %d pairs, %d experts, tiles of %d", n_pairs, n_experts, tile_rows);
   route_sort_kernel<<<1, 1024, 2 * n_experts * sizeof(int), (hipStream_t)stream>>>(experts, n_pairs, n_experts, top, sorted,
-                                                                                  sorted_tokens, tiles, n_tiles, place_of, first_of);
+                                                                                  sorted_tokens, tiles, n_tiles, place_of, first_of, tile_rows);
   AXK_LAUNCH_CHECK("route_sort");
   return 0;
 }

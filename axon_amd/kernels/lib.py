@@ -80,11 +80,11 @@ _SIGNATURES = {
     "axk_clamped_glu": [c_void_p, c_void_p, c_int, c_int, c_float, c_float, c_void_p],
     "axk_grouped_gemm_uses_mfma": [c_int, c_int, c_long, c_long],
     "axk_grouped_gemm": [c_void_p, c_int, c_long, c_long, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_long, c_long,
-                         c_void_p, c_void_p, c_long, c_int, c_float, c_float, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
+                         c_void_p, c_void_p, c_long, c_int, c_float, c_float, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int,
                          c_int, c_void_p],
     "axk_route_topk": [c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p],
-    "axk_route_max_tiles": [c_int, c_int],
-    "axk_route_sort": [c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p],
+    "axk_route_max_tiles": [c_int, c_int, c_int],
+    "axk_route_sort": [c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p],
     "axk_route_combine": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p, c_void_p],
     "axk_gather_rows": [c_void_p, c_long, c_void_p, c_void_p, c_int, c_int, c_void_p],
     "axk_causal_conv": [c_void_p, c_long, c_void_p, c_void_p, c_int, c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_int, c_int,
@@ -690,8 +690,9 @@ class Kernels:
         x [rows, >= g xgs + K] float32 or compute dtype, rows may be strided; w [G, N, K] (with `glu`
         = (limit, alpha): [G, 2 N, K], gate rows then up rows) in the compute dtype; out float32 or
         compute dtype.  Block-diagonal: every row meets every group.  `routed` = (tiles, n_tiles,
-        max_tiles, x_rows, out_rows), int32 on the device: the listed rows (`rows` of them at
-        most) meet the group their tile names.  `gate` (float32, out's shape): out is multiplied
+        max_tiles, x_rows, out_rows[, tile_rows]), int32 on the device: the listed rows (`rows` of them at
+        most) meet the group their tile names; tile_rows (16, or 64: many rows a group) is what the list
+        was made for.  `gate` (float32, out's shape): out is multiplied
         by its sigmoid."""
         G, NW, K = w.shape
         N = NW // 2 if glu else NW
@@ -712,9 +713,10 @@ class Kernels:
             if gate.dtype != torch.float32 or not gate.is_cuda or gate.dim() != 2 or gate.shape[0] != out.shape[0] or gate.stride(-1) != 1:
                 raise KernelError(f"grouped_gemm: gate {tuple(gate.shape)} for out {tuple(out.shape)}")
         tiles = n_tiles = x_rows = out_rows = None
-        max_tiles = 0
+        max_tiles, tile_rows = 0, 16
         if routed is not None:
-            tiles, n_tiles, max_tiles, x_rows, out_rows = routed
+            tiles, n_tiles, max_tiles, x_rows, out_rows = routed[:5]
+            tile_rows = routed[5] if len(routed) > 5 else 16
             for t in (tiles, n_tiles, x_rows, out_rows):
                 if t is not None:
                     self._i32(t, "grouped_gemm routing")
@@ -725,7 +727,7 @@ class Kernels:
             _ptr(x), 1 if x.dtype == torch.float32 else 0, x.stride(0), x_group_stride, _ptr(x_rows), _ptr(w), _ptr(bias),
             self._vec_flag(bias, "grouped bias"), _ptr(out), 1 if out.dtype == torch.float32 else 0, out.stride(0),
             out_group_stride, _ptr(out_rows), _ptr(gate), 0 if gate is None else gate.stride(0), 1 if glu else 0, float(limit),
-            float(alpha), _ptr(tiles), _ptr(n_tiles), int(max_tiles), M, N, K, G, _stream()))
+            float(alpha), _ptr(tiles), _ptr(n_tiles), int(max_tiles), int(tile_rows), M, N, K, G, _stream()))
         return out
 
     # ------------------------------------------------------------------ routing
@@ -736,11 +738,11 @@ class Kernels:
             raise KernelError(f"route_topk: {tuple(experts.shape)} / {tuple(weights.shape)} for {T} x {top}")
         self._check(self.lib.axk_route_topk(_ptr(logits), T, E, top, _ptr(experts), _ptr(weights), _stream()))
 
-    def route_max_tiles(self, n_pairs: int, n_experts: int) -> int:
-        return int(self.lib.axk_route_max_tiles(n_pairs, n_experts))
+    def route_max_tiles(self, n_pairs: int, n_experts: int, tile_rows: int = 16) -> int:
+        return int(self.lib.axk_route_max_tiles(n_pairs, n_experts, tile_rows))
 
     def route_sort(self, experts: torch.Tensor, n_experts: int, sorted_pairs, sorted_tokens, tiles, n_tiles, place_of=None,
-                   first_of=None) -> None:
+                   first_of=None, tile_rows: int = 16) -> None:
         """The pairs in expert order, their tokens, the grouped product's tiles; optionally where each
         pair stands (place_of [pairs]) and where each expert's pairs start (first_of [experts + 1])."""
         for t in (experts, sorted_pairs, sorted_tokens, tiles, n_tiles) + tuple(t for t in (place_of, first_of) if t is not None):
@@ -748,10 +750,10 @@ class Kernels:
         if (place_of is not None and place_of.numel() < experts.numel()) or (first_of is not None and first_of.numel() < n_experts + 1):
             raise KernelError("route_sort: place_of or first_of is too short")
         P = experts.numel()
-        if sorted_pairs.numel() < P or sorted_tokens.numel() < P or tiles.numel() < 3 * self.route_max_tiles(P, n_experts):
+        if sorted_pairs.numel() < P or sorted_tokens.numel() < P or tiles.numel() < 3 * self.route_max_tiles(P, n_experts, tile_rows):
             raise KernelError(f"route_sort: lists too short for {P} pairs of {n_experts} experts")
         self._check(self.lib.axk_route_sort(_ptr(experts), P, n_experts, experts.shape[-1], _ptr(sorted_pairs), _ptr(sorted_tokens),
-                                            _ptr(tiles), _ptr(n_tiles), _ptr(place_of), _ptr(first_of), _stream()))
+                                            _ptr(tiles), _ptr(n_tiles), _ptr(place_of), _ptr(first_of), int(tile_rows), _stream()))
 
     def gather_rows(self, x: torch.Tensor, rows: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
         self._elem(x, "gather x"); self._elem(out, "gather out"); self._i32(rows, "gather rows")

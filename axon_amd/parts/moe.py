@@ -5,11 +5,9 @@ Router logits are 32-bit (Wr h with h in the compute dtype).  An expert is a gat
 clamps: g = min(Wgate h, limit), u = clamp(Wup h, -limit, limit), out = Wdown (g sigmoid(alpha g)
 (u + 1)), without biases.  The (token, chosen expert) pairs are listed expert by expert on the
 device and two grouped products (gate|up with the activation in its epilogue, then down) run
-over the list; a token's rows are then added in the order of its router's ranking.  A step with
-many rows an expert (a long prompt) instead reads where each expert's rows start, brings the rows
-into expert order and gives every expert's stretch to the engine's large products, matrix by
-matrix: the one place where the host waits for the device inside a step, worth it from some 64
-rows an expert on; steps of single tokens never take it (a captured graph could not).
+over the list; a token's rows are then added in the order of its router's ranking.  With many rows
+an expert (a long prompt) the list is made in tiles of 64 rows, which the grouped product takes
+through LDS: the same chains and bits as the tiles of 16 of a short step.
 
 Parameters: `hidden_size`, `experts`, `top`, `ff`, `limit`, `alpha` (default 1.702), `shared`
 (None, or {"ff", "limit"}), `names` (scope "mlp.", router, expert "e{}.", shared "shared.").
@@ -21,7 +19,7 @@ from typing import List
 import torch
 
 from ..config.base import ConfigError, PartSpec
-from ..kernels import MODE_STORE, MODE_STORE_F32
+from ..kernels import MODE_STORE_F32
 from .base import FeedForward, TensorDecl, build_part, register_feed_forward
 
 
@@ -72,30 +70,6 @@ class RoutedExperts(FeedForward):
                 store.forget(self._expert(e, which))
         if self.shared is not None:
             self.shared.load(store, rt)
-        # the same matrices one by one, as the large products want them (packed where they can be)
-        self.by_expert = [(rt.k.prepare_weight(self.w_gate_up[e]), rt.k.prepare_weight(self.w_down[e])) for e in range(E)]
-
-    ROWS_AN_EXPERT = 64        # from this many rows an expert on average, a step goes expert by expert
-
-    def _expert_by_expert(self, ctx, h, out, accumulate, chosen, weights) -> None:
-        k, T, E, top = ctx.rt.k, h.shape[0], self.n_experts, self.top
-        i32, P = torch.int32, h.shape[0] * self.top
-        pairs, tokens, place_of = ctx.ws.take((P,), i32), ctx.ws.take((P,), i32), ctx.ws.take((P,), i32)
-        tiles, n_tiles = ctx.ws.take((3 * k.route_max_tiles(P, E),), i32), ctx.ws.take((1,), i32)
-        first_of = ctx.ws.take((E + 1,), i32)
-        k.route_sort(chosen, E, pairs, tokens, tiles, n_tiles, place_of, first_of)
-        first = first_of.tolist()                                # the host waits here
-        x = k.gather_rows(h, tokens, ctx.ws.take((P, self.hidden), ctx.rt.dtype))
-        gate_up = ctx.ws.take((P, 2 * self.ff), ctx.rt.dtype)
-        for e, (w, _) in enumerate(self.by_expert):
-            if first[e + 1] > first[e]:
-                k.gemm(x[first[e]:first[e + 1]], w, gate_up[first[e]:first[e + 1]], None, MODE_STORE)
-        act = k.clamped_glu(gate_up, ctx.ws.take((P, self.ff), ctx.rt.dtype), self.limit, self.alpha)
-        rows = ctx.ws.take((P, self.hidden), torch.float32)
-        for e, (_, w) in enumerate(self.by_expert):
-            if first[e + 1] > first[e]:
-                k.gemm(act[first[e]:first[e + 1]], w, rows[first[e]:first[e + 1]], None, MODE_STORE_F32)
-        k.route_combine(rows, weights, out, accumulate, place_of)
 
     def forward(self, ctx, h, out, accumulate: bool = True) -> None:
         k, T, E, top = ctx.rt.k, h.shape[0], self.n_experts, self.top
@@ -104,22 +78,18 @@ class RoutedExperts(FeedForward):
         k.gemm(h, self.w_router, logits, None, MODE_STORE_F32)
         chosen, weights = ctx.ws.take((T, top), i32), ctx.ws.take((T, top), torch.float32)
         k.route_topk(logits, top, chosen, weights)
-        if not ctx.decode_only and T * top >= self.ROWS_AN_EXPERT * E:
-            self._expert_by_expert(ctx, h, out, accumulate, chosen, weights)
-            if self.shared is not None:
-                self.shared.forward(ctx, h, out)
-            return
         P = T * top
-        max_tiles = k.route_max_tiles(P, E)
+        tile_rows = 64 if P >= 32 * E else 16          # many rows an expert: tiles of 64 rows through LDS (the same bits)
+        max_tiles = k.route_max_tiles(P, E, tile_rows)
         pairs, tokens = ctx.ws.take((P,), i32), ctx.ws.take((P,), i32)
         tiles, n_tiles = ctx.ws.take((3 * max_tiles,), i32), ctx.ws.take((1,), i32)
-        k.route_sort(chosen, E, pairs, tokens, tiles, n_tiles)
+        k.route_sort(chosen, E, pairs, tokens, tiles, n_tiles, tile_rows=tile_rows)
         act = ctx.ws.take((P, self.ff), ctx.rt.dtype)
         k.grouped_gemm(h, self.w_gate_up, act, x_group_stride=0, out_group_stride=0, glu=(self.limit, self.alpha),
-                       routed=(tiles, n_tiles, max_tiles, tokens, pairs), rows=P)
+                       routed=(tiles, n_tiles, max_tiles, tokens, pairs, tile_rows), rows=P)
         rows = ctx.ws.take((P, self.hidden), torch.float32)
         k.grouped_gemm(act, self.w_down, rows, x_group_stride=0, out_group_stride=0,
-                       routed=(tiles, n_tiles, max_tiles, pairs, pairs), rows=P)
+                       routed=(tiles, n_tiles, max_tiles, pairs, pairs, tile_rows), rows=P)
         k.route_combine(rows, weights, out, accumulate)
         if self.shared is not None:
             self.shared.forward(ctx, h, out)

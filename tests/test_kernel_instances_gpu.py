@@ -383,6 +383,8 @@ CASES = [
     (BF, ["grouped_gemm<1,1>"], check_grouped, (BF, 19, 2, 72, 160, True)),
     (BF, ["grouped_gemm<0,0>"], check_grouped, (BF, 50, 3, 40, 24, False)),
     (BF, ["grouped_gemm<0,1>"], check_grouped, (BF, 19, 2, 72, 40, True)),
+    (BF, ["grouped_gemm<2,0>"], check_grouped, (BF, 300, 3, 40, 64, False)),       # many rows: tiles of 64 through LDS
+    (BF, ["grouped_gemm<2,1>"], check_grouped, (BF, 270, 2, 72, 160, True)),
     (F32, ["grouped_gemm<0,0>"], check_grouped, (F32, 50, 3, 40, 64, False)),
     (F32, ["grouped_gemm<0,1>"], check_grouped, (F32, 19, 2, 72, 160, True)),
     # attention on the matrix cores: (head size, query heads a block, pages of 64 positions or more)

@@ -443,6 +443,25 @@ def test_grouped_products_block_diagonal_and_routed(dtype):
     act = torch.zeros(P_, F, dtype=td, device="cuda")
     k.grouped_gemm(h.to(td).cuda(), w.to(td).cuda(), act, x_group_stride=0, out_group_stride=0, glu=(1.2, 1.702),
                    routed=(tiles, n_tiles, max_tiles, tokens, pairs), rows=P_)
+    # the same rows listed in tiles of 64 (many rows a group): the same bits; and what else the listing offers
+    wide_tiles, n_wide = torch.zeros(3 * k.route_max_tiles(P_, E, 64), dtype=torch.int32, device="cuda"), torch.zeros(1, dtype=torch.int32, device="cuda")
+    pairs64, tokens64 = torch.zeros_like(pairs), torch.zeros_like(tokens)
+    place_of, first_of = torch.zeros(P_, dtype=torch.int32, device="cuda"), torch.zeros(E + 1, dtype=torch.int32, device="cuda")
+    k.route_sort(chosen, E, pairs64, tokens64, wide_tiles, n_wide, place_of, first_of, tile_rows=64)
+    assert int(n_wide) <= E and pairs64[place_of.long()].tolist() == list(range(P_))
+    assert first_of.tolist() == [0] + torch.bincount(idx.view(-1), minlength=E).cumsum(0).tolist()
+    act64 = torch.zeros(P_, F, dtype=td, device="cuda")
+    k.grouped_gemm(h.to(td).cuda(), w.to(td).cuda(), act64, x_group_stride=0, out_group_stride=0, glu=(1.2, 1.702),
+                   routed=(wide_tiles, n_wide, k.route_max_tiles(P_, E, 64), tokens64, pairs64, 64), rows=P_)
+    assert torch.equal(act64, act)
+    gathered = k.gather_rows(h.to(td).cuda(), tokens64, torch.zeros(P_, K, dtype=td, device="cuda"))
+    assert torch.equal(gathered.cpu(), h.to(td)[tokens64.cpu().long()])
+    rows32 = torch.randn(P_, 8, generator=g).cuda()
+    y_a, y_b = torch.zeros(T, 8, device="cuda"), torch.zeros(T, 8, device="cuda")
+    k.route_combine(rows32, weights, y_a)
+    k.route_combine(rows32[pairs64.long()].contiguous(), weights, y_b, place_of=place_of)
+    assert torch.equal(y_a, y_b)
+    assert float((y_a.cpu() - (rows32.cpu().view(T, top, 8) * weights.cpu()[:, :, None]).sum(1)).abs().max()) < 1e-5
     for p in range(P_):
         e = int(idx.view(-1)[p])
         z = h[p // top].double() @ w[e].double().T
