@@ -306,24 +306,24 @@ latent_attention_mfma_kernel(const float* __restrict__ q_full, const bf16_t* __r
 }
 
 // o_lat[row, :] = sum_c exp(m_c - M) o_c / sum_c exp(m_c - M) l_c over a row's blocks in ascending order
-// (M the largest m_c; a block that saw nothing has l = 0 and is skipped).  One block per (token, head).
-__global__ void latent_attention_fold_kernel(const float* __restrict__ partial, float* __restrict__ o_lat, int rank, int n_chunks) {
+// (M the largest m_c; a block that saw nothing has l = 0 and weighs nothing).  One block per (token,
+// head): the blocks' weights once into LDS, then a thread a dim.
+__global__ void __launch_bounds__(128)
+latent_attention_fold_kernel(const float* __restrict__ partial, float* __restrict__ o_lat, int rank, int n_chunks) {
+  extern __shared__ float weight[];
   const float* src = partial + (long)blockIdx.x * n_chunks * (rank + 2);
   float M = -INFINITY;
   for (int c = 0; c < n_chunks; ++c)
     if (src[(long)c * (rank + 2) + rank + 1] > 0.0f) M = fmaxf(M, src[(long)c * (rank + 2) + rank]);
+  for (int c = threadIdx.x; c < n_chunks; c += blockDim.x)
+    weight[c] = src[(long)c * (rank + 2) + rank + 1] > 0.0f ? expf(src[(long)c * (rank + 2) + rank] - M) : 0.0f;
+  __syncthreads();
   float L = 0.0f;
-  for (int c = 0; c < n_chunks; ++c) {
-    const float l = src[(long)c * (rank + 2) + rank + 1];
-    if (l > 0.0f) L = fmaf(expf(src[(long)c * (rank + 2) + rank] - M), l, L);
-  }
+  for (int c = 0; c < n_chunks; ++c) L = fmaf(weight[c], src[(long)c * (rank + 2) + rank + 1], L);
   const float inv = 1.0f / L;
   for (int d = threadIdx.x; d < rank; d += blockDim.x) {
     float o = 0.0f;
-    for (int c = 0; c < n_chunks; ++c) {
-      const float l = src[(long)c * (rank + 2) + rank + 1];
-      if (l > 0.0f) o = fmaf(expf(src[(long)c * (rank + 2) + rank] - M), src[(long)c * (rank + 2) + d], o);
-    }
+    for (int c = 0; c < n_chunks; ++c) o = fmaf(weight[c], src[(long)c * (rank + 2) + d], o);
     o_lat[(long)blockIdx.x * rank + d] = o * inv;
   }
 }
@@ -337,7 +337,7 @@ static void launch_latent_mfma(const float* q_full, const void* cache, const int
   latent_attention_mfma_kernel<RT, QC><<<grid, LAM_WAVES * 64, 0, stream>>>(
       q_full, (const bf16_t*)cache, block_table, table_stride, positions, seq_rows, o_lat, n_tokens, heads, rank, rot, page_size,
       window, scale, partial, n_chunks);
-  if (partial) latent_attention_fold_kernel<<<n_tokens * heads, 128, 0, stream>>>(partial, o_lat, rank, n_chunks);
+  if (partial) latent_attention_fold_kernel<<<n_tokens * heads, 128, n_chunks * sizeof(float), stream>>>(partial, o_lat, rank, n_chunks);
 }
 #endif
 

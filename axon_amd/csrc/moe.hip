@@ -36,6 +36,40 @@ __global__ void route_topk_kernel(const float* __restrict__ logits, int n_tokens
   for (int k = 0; k < top; ++k) w[k] = w[k] / sum;
 }
 
+// The same choice by a wave per token (up to 1,024 experts: lane l holds the logits of experts l, l + 64, ...):
+// `top` times the largest logit not yet taken, by a butterfly over (logit, lower expert first).
+__global__ void route_topk_wave_kernel(const float* __restrict__ logits, int n_tokens, int n_experts, int top,
+                                       int32_t* __restrict__ experts, float* __restrict__ weights) {
+  const int t = blockIdx.x * (blockDim.x / 64) + threadIdx.x / 64, lane = threadIdx.x & 63;
+  if (t >= n_tokens) return;
+  float z[16];
+#pragma unroll
+  for (int i = 0; i < 16; ++i) z[i] = lane + 64 * i < n_experts ? logits[(long)t * n_experts + lane + 64 * i] : -INFINITY;
+  unsigned taken = 0;
+  float first = 0.0f, sum = 0.0f, mine = 0.0f;        // lane k keeps the k-th weight
+  for (int k = 0; k < top; ++k) {
+    float best = -INFINITY;
+    int at = 0x7fffffff;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      const int e = lane + 64 * i;
+      if (e < n_experts && !(taken >> i & 1) && (at == 0x7fffffff || z[i] > best)) { best = z[i]; at = e; }
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+      const float other = __shfl_xor(best, off, 64);
+      const int other_at = __shfl_xor(at, off, 64);
+      if (other_at != 0x7fffffff && (at == 0x7fffffff || other > best || (other == best && other_at < at))) { best = other; at = other_at; }
+    }
+    if ((at & 63) == lane) taken |= 1u << (at >> 6);
+    if (k == 0) first = best;
+    const float p = expf(best - first);
+    sum += p;
+    if (lane == k % 64) { mine = p; experts[(long)t * top + k] = at; }
+  }
+  if (lane < top) weights[(long)t * top + lane] = mine / sum;
+}
+
 // One block.  pairs p = t top + k in expert order -> sorted [n_pairs], with the token of each
 // (sorted_tokens); tiles [.][3] = (expert, first place in sorted, count <= tile_rows), *n_tiles of them.
 // Which place a pair gets inside its expert's stretch is not fixed (atomic counters); no result
@@ -104,6 +138,11 @@ extern "C" int axk_route_topk(const float* logits, int n_tokens, int n_experts, 
   AXK_REQUIRE(n_tokens >= 0 && n_experts > 0 && top > 0 && top <= n_experts, "route_topk: %d tokens, %d of %d experts",
               n_tokens, top, n_experts);
   if (n_tokens == 0) return 0;
+  if (n_experts <= 1024 && top <= 64) {
+    route_topk_wave_kernel<<<ceil_div(n_tokens, 4), 256, 0, (hipStream_t)stream>>>(logits, n_tokens, n_experts, top, experts, weights);
+    AXK_LAUNCH_CHECK("route_topk");
+    return 0;
+  }
   route_topk_kernel<<<ceil_div(n_tokens, 64), 64, 0, (hipStream_t)stream>>>(logits, n_tokens, n_experts, top, experts, weights);
   AXK_LAUNCH_CHECK("route_topk");
   return 0;

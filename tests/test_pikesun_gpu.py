@@ -430,6 +430,17 @@ def test_grouped_products_block_diagonal_and_routed(dtype):
     val, idx = torch.topk(logits, top, dim=-1)
     assert torch.equal(chosen.cpu().long(), idx)
     assert float((weights.cpu() - torch.softmax(val, -1)).abs().max()) < 1e-6
+    for n_e, n_top, rows_ in ((200, 7, 33), (64, 64, 3), (1100, 3, 9)):          # a wave a token; every expert; a thread a token
+        z = torch.randn(rows_, n_e, generator=g)
+        c2, w2 = torch.zeros(rows_, n_top, dtype=torch.int32, device="cuda"), torch.zeros(rows_, n_top, dtype=torch.float32, device="cuda")
+        k.route_topk(z.cuda(), n_top, c2, w2)
+        v2, i2 = torch.topk(z, n_top, dim=-1)
+        assert torch.equal(c2.cpu().long(), i2) and float((w2.cpu() - torch.softmax(v2, -1)).abs().max()) < 1e-6
+    tie = torch.zeros(2, 70)
+    tie[:, [3, 9, 68]] = 1.0
+    c2, w2 = torch.zeros(2, 2, dtype=torch.int32, device="cuda"), torch.zeros(2, 2, dtype=torch.float32, device="cuda")
+    k.route_topk(tie.cuda(), 2, c2, w2)
+    assert c2.tolist() == [[3, 9], [3, 9]] and w2.tolist() == [[0.5, 0.5], [0.5, 0.5]]      # of equal logits the lower expert
     P_ = T * top
     pairs, tokens = torch.zeros(P_, dtype=torch.int32, device="cuda"), torch.zeros(P_, dtype=torch.int32, device="cuda")
     max_tiles = k.route_max_tiles(P_, E)
