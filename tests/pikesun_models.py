@@ -68,6 +68,17 @@ MODELS = {
         layer(att(heads=2, dim=16, rot_dim=8, vdim=8, kv_rank=24, q_rank=40, window=0), dense(64)),
         layer(att(heads=5, dim=8, rot_dim=2, vdim=16, kv_rank=12, q_rank=8, window=33, scale=0.8), moe(3, 2, 16, 0.7))],
         eps=1e-4, mult=1.3, scale=9.0), page=16, seed=5),
+    # recurrences only: no pages at all, a layer without a feed-forward between two that share tensors
+    "S": dict(cfg=config(80, 140, [
+        layer(rec(96, 4, 4), moe(5, 3, 24, 1.2)),
+        layer(rec(160, 2, 2), None),
+        layer(rec(96, 4, 4), moe(5, 3, 24, 1.2), weights_of=0)], eps=1e-6, mult=0.8, scale=2.0), page=32, seed=12),
+    # sixteen heads and latents in sixteens: the matrix-core attention inside a whole model, with pages of 64
+    "T": dict(cfg=config(64, 190, [
+        layer(att(heads=16, dim=16, rot_dim=16, vdim=8, kv_rank=48, q_rank=32, window=75), dense(96)),
+        layer(rec(64, 2, 3), moe(4, 2, 32, 2.0, (32, 2.0))),
+        layer(att(heads=16, dim=16, rot_dim=16, vdim=8, kv_rank=48, q_rank=32, window=75), dense(96), weights_of=0)],
+        eps=1e-5, mult=0.9, scale=3.0), page=64, seed=14),
 }
 
 

@@ -43,6 +43,11 @@ def test_two_attention_layers_of_other_sizes_get_pools_of_their_own():
     assert [(s.head_dim, s.window) for s in plan.group_specs] == [(56, 0), (26, 33)] and plan.state_elems == [(2 * 64, "float32")]
 
 
+def test_a_model_of_recurrences_alone_has_no_pages():
+    plan = build_model_description(config_from_dict(MODELS["S"]["cfg"])).cache_plan
+    assert plan.group_specs == [] and [e for e, _ in plan.state_elems] == [2 * 4 * 96, 2 * 2 * 160, 2 * 4 * 96]
+
+
 def test_a_layer_without_a_feed_forward_and_defaults():
     cfg = config(32, 50, [layer(rec(32, 2, 2), None)])
     del cfg["embedding"], cfg["residual_mult"]
@@ -120,3 +125,18 @@ def test_plain_mixers_behave_as_the_design_says():
     assert torch.allclose(P.gated_recurrence(W, "l1.mix.", r, later)[:9], out[:9])
     a = torch.exp(-8.0 * torch.log1p(torch.exp(W["l1.mix.lam"])))        # r = 1: the fastest decay
     assert float(a.min()) > 0 and float(a.max()) < 1
+
+
+def test_the_command_line_writes_and_describes_a_model_of_the_design(tmp_path, capsys):
+    import json
+    from axon_amd.cli import main
+    cfg_path = tmp_path / "config.json"
+    cfg_path.write_text(json.dumps(MODELS["R"]["cfg"]))
+    out = tmp_path / "model"
+    assert main(["random-weights", str(cfg_path), str(out), "--seed", "3"]) == 0
+    assert main(["info", str(out)]) == 0
+    text = capsys.readouterr().out
+    assert "architecture: Pikesun" in text and "cache group: 1 layers x 1 x 1 heads x 56" in text and "window 33" in text
+    from safetensors.torch import load_file
+    names = set(load_file(str(out / "model.safetensors")))
+    assert names == set(draw_weights(MODELS["R"]["cfg"], 0))
