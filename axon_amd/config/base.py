@@ -104,10 +104,13 @@ class LayerSpec:
 class Run:
     """One entry of the execution order: run `layer` with the cache `cache`.  Two runs may name
     the same layer (its weights are used twice); a run whose `cache` is another run's, with
-    `writes_cache` false, reads what that run wrote and stores nothing of its own."""
+    `writes_cache` false, reads what that run wrote and stores nothing of its own.  `enter`: the
+    index of one of the model's `entries`, a part that rewrites the residual stream right before
+    this run (from the stream and the embedding's output), or None."""
     layer: int
     cache: int
     writes_cache: bool = True
+    enter: Optional[int] = None
 
 
 @dataclass(frozen=True)
@@ -121,6 +124,7 @@ class ModelSpec:
     final_norm: PartSpec
     head: PartSpec
     max_positions: int
+    entries: tuple = ()         # PartSpecs of kind "stream": what runs may `enter` through
 
 
 class ModelConfig:

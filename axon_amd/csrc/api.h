@@ -204,7 +204,9 @@ int axk_norm_add(const float* y, const void* gain, int gain_is_f32, float eps, f
                  int n_rows, int dim, void* stream);
 // out[i] = x[i] in the compute dtype.
 int axk_round_rows(const float* x, void* out, long n, void* stream);
-// In place on elem values; kind 0: the tanh form of GELU.
+// out[t, :] = [a[t, :] | b[t, :]] in the compute dtype (a [n_rows, wa], b [n_rows, wb] float32).
+int axk_concat_round(const float* a, int wa, const float* b, int wb, void* out, int n_rows, void* stream);
+// In place on elem values; kind 0: the tanh form of GELU; kind 1: the exact (erf) GELU.
 int axk_activation(void* v, long n, int kind, void* stream);
 // out[t, f] = g sigmoid(alpha g) (u + 1), g = min(gate_up[t, f], limit), u = clamp(gate_up[t, F + f], -limit, limit).
 int axk_clamped_glu(const void* gate_up, void* out, int n_tokens, int n_ffn, float limit, float alpha, void* stream);
@@ -289,6 +291,33 @@ long axk_latent_attention_workspace(int n_tokens, int heads, int rank, int rot, 
 int axk_latent_attention(const float* q_full, const void* cache, const int32_t* block_table, int table_stride,
                          const int32_t* positions, const int32_t* seq_rows, float* o_lat, int n_tokens, int heads, int rank,
                          int rot, int page_size, int window, float scale, float* partial, long partial_floats, void* stream);
+
+// Grouped-query attention with one or two score maps a head, an optional norm of queries and keys, a
+// sliding-window or chunked mask, bent scores and a gate (csrc/masked_attention.hip).  A page is
+// [page_size][kv_heads maps dim] elem (key rows), then [kv_heads vdim][page_size] (values, the positions
+// of one dim side by side).
+// axk_heads_prepare: from the float32 rows of the projections (n_q query units and n_k key units of `dim`
+// each, v_width values; v_at may equal k_at), units RMS-normed with a gain shared by all units (null: no
+// norm), the first `rot` dims rotated by table [T, rot / 2, 2] (sin, cos; both scaled by `magnitude`) in
+// pairs (2i, 2i + 1) if `neighbours` else (i, i + rot / 2); queries into q_out elem [T, n_q dim], keys and
+// values into the page (if write_kv).
+int axk_heads_prepare(const float* proj, long stride, int q_at, int n_q, int k_at, int n_k, int v_at, int v_width, int dim,
+                      const void* q_gain, int q_gain_is_f32, const void* k_gain, int k_gain_is_f32, float eps, int rot,
+                      int neighbours, float magnitude, const float* table, const int32_t* positions, const int32_t* seq_rows,
+                      const int32_t* block_table, int table_stride, void* cache, int page_size, void* q_out, int n_tokens,
+                      int write_kv, void* stream);
+// axk_masked_attention: q elem [T, heads maps dim] -> out elem [T, heads vdim].  mask_kind 0: all earlier
+// positions; 1: the last mask_size positions; 2: the earlier positions of the same chunk of mask_size.
+// softcap > 0: s <- softcap tanh(s / softcap).  maps 2: o = rms(a_1 - lambda a_2, eps) out_scale.  gate
+// (float32 rows of gate_stride, or null): o *= sigmoid(gate).  tiles (int32 [n_tiles, 2]: first token,
+// count; up to 16 consecutive tokens of one request each) or null (every token a tile of its own) are
+// what the matrix-core kernel works on where axk_masked_attention_uses_mfma says 1.
+int axk_masked_attention_uses_mfma(int heads, int kv_heads, int maps, int dim, int vdim, int page_size);
+int axk_masked_attention(const void* q, const void* cache, const int32_t* block_table, int table_stride,
+                         const int32_t* positions, const int32_t* seq_rows, const float* gate, long gate_stride, void* out,
+                         int n_tokens, int heads, int kv_heads, int maps, int dim, int vdim, int page_size, int mask_kind,
+                         int mask_size, float scale, float softcap, float lambda, float out_scale, float eps,
+                         const int32_t* tiles, int n_tiles, void* stream);
 
 #ifdef __cplusplus
 }

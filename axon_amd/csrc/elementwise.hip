@@ -298,18 +298,44 @@ extern "C" int axk_round_rows(const float* x, void* out, long n, void* stream) {
   return 0;
 }
 
+// Two row sets side by side in the compute dtype: out[t, :wa] = a[t, :], out[t, wa:] = b[t, :].
+__global__ void concat_round_kernel(const float* __restrict__ a, int wa, const float* __restrict__ b, int wb,
+                                    elem_t* __restrict__ out) {
+  const long t = blockIdx.y;
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= wa + wb) return;
+  out[t * (wa + wb) + i] = from_float(i < wa ? a[t * wa + i] : b[t * wb + i - wa]);
+}
+
+extern "C" int axk_concat_round(const float* a, int wa, const float* b, int wb, void* out, int n_rows, void* stream) {
+  AXK_REQUIRE(n_rows >= 0 && n_rows <= 65535 * 64 && wa > 0 && wb > 0, "concat_round: bad sizes rows=%d widths %d and %d", n_rows, wa, wb);
+  if (n_rows == 0) return 0;
+  for (int r0 = 0; r0 < n_rows; r0 += 65535) {
+    const int rows = n_rows - r0 < 65535 ? n_rows - r0 : 65535;
+    concat_round_kernel<<<dim3((wa + wb + 255) / 256, rows), 256, 0, (hipStream_t)stream>>>(
+        a + (long)r0 * wa, wa, b + (long)r0 * wb, wb, (elem_t*)out + (long)r0 * (wa + wb));
+  }
+  AXK_LAUNCH_CHECK("concat_round");
+  return 0;
+}
+
 // ---------------------------------------------------------------------------- activations
-// kind 0: the tanh form of GELU, 0.5 z (1 + tanh(sqrt(2 / pi) (z + 0.044715 z^3))), in place.
+// In place.  kind 0: the tanh form of GELU, 0.5 z (1 + tanh(sqrt(2 / pi) (z + 0.044715 z^3)));
+// kind 1: the exact GELU, 0.5 z (1 + erf(z / sqrt 2)).
 __global__ void activation_kernel(elem_t* __restrict__ v, long n, int kind) {
   const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= n) return;
   const float z = to_float(v[i]);
+  if (kind == 1) {
+    v[i] = from_float((0.5f * z) * (1.0f + erff(z * 0.7071067811865476f)));
+    return;
+  }
   const float inner = 0.7978845608028654f * (z + 0.044715f * ((z * z) * z));
   v[i] = from_float((0.5f * z) * (1.0f + tanhf(inner)));
 }
 
 extern "C" int axk_activation(void* v, long n, int kind, void* stream) {
-  AXK_REQUIRE(kind == 0, "activation: kind %d is not known (0: gelu, tanh form)", kind);
+  AXK_REQUIRE(kind == 0 || kind == 1, "activation: kind %d is not known (0: gelu, tanh form; 1: gelu, exact)", kind);
   if (n <= 0) return 0;
   activation_kernel<<<(unsigned)((n + 255) / 256), 256, 0, (hipStream_t)stream>>>((elem_t*)v, n, kind);
   AXK_LAUNCH_CHECK("activation");

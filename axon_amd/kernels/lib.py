@@ -96,6 +96,14 @@ _SIGNATURES = {
     "axk_latent_query_rope": [c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],
     "axk_latent_attention": [c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
                              c_int, c_int, c_float, c_void_p, c_long, c_void_p],
+    "axk_heads_prepare": [c_void_p, c_long, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_int, c_void_p, c_int, c_float,
+                          c_int, c_int, c_float, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p, c_int,
+                          c_int, c_void_p],
+    "axk_masked_attention_uses_mfma": [c_int, c_int, c_int, c_int, c_int, c_int],
+    "axk_masked_attention": [c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_long, c_void_p, c_int, c_int,
+                             c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_float, c_float, c_float, c_float,
+                             c_void_p, c_int, c_void_p],
+    "axk_concat_round": [c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_void_p],
     "axk_fill_i32": [c_void_p, c_int, c_int, c_void_p],
     "axk_fill_f32": [c_void_p, c_float, c_int, c_void_p],
 }
@@ -208,7 +216,7 @@ class Kernels:
                   "attention_decode", "gemm", "gemm_normed_glu", "gemm_normed_qkv_rope", "swiglu", "argmax", "topk",
                   "fill_i32", "fill_f32", "call", "norm_add", "round_rows", "activation", "clamped_glu", "grouped_gemm",
                   "route_topk", "route_sort", "route_combine", "gather_rows", "causal_conv", "gated_scan", "latent_prepare",
-                  "latent_query_rope", "latent_attention")
+                  "latent_query_rope", "latent_attention", "heads_prepare", "masked_attention", "concat_round")
     _MATRIX_AT = {"gemm": 1, "gemm_qkv_rope": 1, "gemm_normed_glu": 3, "gemm_normed_qkv_rope": 3, "grouped_gemm": 1}   # which argument is W
 
     def set_launch_hook(self, hook) -> None:
@@ -666,12 +674,23 @@ class Kernels:
         self._check(self.lib.axk_round_rows(_ptr(x), _ptr(out), x.numel(), _stream()))
         return out
 
+    ACTIVATIONS = {"gelu_tanh": 0, "gelu_erf": 1}
+
     def activation(self, v: torch.Tensor, kind: str = "gelu_tanh") -> torch.Tensor:
         self._elem(v, "activation")
-        if kind != "gelu_tanh" or not v.is_contiguous():
+        if kind not in self.ACTIVATIONS or not v.is_contiguous():
             raise KernelError(f"activation: '{kind}' on a tensor of strides {v.stride()}")
-        self._check(self.lib.axk_activation(_ptr(v), v.numel(), 0, _stream()))
+        self._check(self.lib.axk_activation(_ptr(v), v.numel(), self.ACTIVATIONS[kind], _stream()))
         return v
+
+    def concat_round(self, a: torch.Tensor, b: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+        """out = [a | b] row by row, rounded to the compute dtype."""
+        self._f32(a, "concat_round a"); self._f32(b, "concat_round b"); self._elem(out, "concat_round out")
+        if a.dim() != 2 or b.dim() != 2 or a.shape[0] != b.shape[0] or out.shape != (a.shape[0], a.shape[1] + b.shape[1]) \
+                or not out.is_contiguous():
+            raise KernelError(f"concat_round: {tuple(a.shape)} and {tuple(b.shape)} into {tuple(out.shape)}")
+        self._check(self.lib.axk_concat_round(_ptr(a), a.shape[1], _ptr(b), b.shape[1], _ptr(out), a.shape[0], _stream()))
+        return out
 
     def clamped_glu(self, gate_up: torch.Tensor, out: torch.Tensor, limit: float, alpha: float) -> torch.Tensor:
         self._elem(gate_up, "clamped_glu in"); self._elem(out, "clamped_glu out")
@@ -862,6 +881,66 @@ class Kernels:
                                                   _ptr(positions), _ptr(seq_rows), _ptr(o_lat), T, heads, rank, rot, page_size,
                                                   int(window), float(scale), _ptr(partial), need, _stream()))
         return o_lat
+
+    # ------------------------------------------------------------------ attention with maps, masks and bent scores
+    MASKS = {"causal": 0, "window": 1, "chunk": 2}
+
+    def _check_heads_cache(self, cache, page_size, row, what) -> None:
+        self._elem(cache, what + " cache")
+        if cache.dim() != 4 or tuple(cache.shape[1:]) != (1, page_size, row) or not cache.is_contiguous():
+            raise KernelError(f"{what}: cache {tuple(cache.shape)} is not [pages, 1, {page_size}, {row}]")
+
+    def heads_prepare(self, proj, q_at, n_q, k_at, n_k, v_at, v_width, dim, q_gain, k_gain, eps, rot, neighbours, magnitude,
+                      table, positions, seq_rows, block_table, cache, page_size, q_out, write_kv=True) -> None:
+        """The projections' float32 rows into queries (q_out) and the page's keys and values: see
+        axk_heads_prepare in csrc/api.h."""
+        self._f32(proj, "heads proj"); self._f32(table, "rope table"); self._i32(positions, "positions")
+        self._i32(seq_rows, "seq_rows"); self._i32(block_table, "block_table"); self._elem(q_out, "heads q_out")
+        T = positions.numel()
+        if proj.dim() != 2 or proj.shape[0] != T or (rot and table.shape != (T, rot // 2, 2)) or seq_rows.numel() != T:
+            raise KernelError(f"heads_prepare: proj {tuple(proj.shape)}, table {tuple(table.shape)} for {T} tokens")
+        self._check_heads_cache(cache, page_size, n_k * dim + v_width, "heads_prepare")
+        if q_out.shape != (T, n_q * dim) or not q_out.is_contiguous():
+            raise KernelError(f"heads_prepare: q_out {tuple(q_out.shape)} is not [{T}, {n_q * dim}]")
+        for gain in (q_gain, k_gain):
+            if gain is not None and gain.numel() != dim:
+                raise KernelError(f"heads_prepare: a gain of {gain.numel()} for units of {dim}")
+        self._check(self.lib.axk_heads_prepare(
+            _ptr(proj), proj.stride(0), q_at, n_q, k_at, n_k, v_at, v_width, dim, _ptr(q_gain), self._vec_flag(q_gain, "q gain"),
+            _ptr(k_gain), self._vec_flag(k_gain, "k gain"), float(eps), rot, 1 if neighbours else 0, float(magnitude), _ptr(table),
+            _ptr(positions), _ptr(seq_rows), _ptr(block_table), block_table.shape[-1], _ptr(cache), page_size, _ptr(q_out), T,
+            1 if write_kv else 0, _stream()))
+
+    def masked_attention_uses_mfma(self, heads, kv_heads, maps, dim, vdim, page_size) -> bool:
+        return bool(self.lib.axk_masked_attention_uses_mfma(heads, kv_heads, maps, dim, vdim, page_size))
+
+    def masked_attention(self, q, cache, block_table, positions, seq_rows, out, heads, kv_heads, maps, dim, vdim, page_size,
+                         mask, mask_size, scale, softcap=0.0, lam=0.0, out_scale=1.0, eps=0.0, gate=None, tiles=None) -> torch.Tensor:
+        """q [T, heads maps dim] -> out [T, heads vdim] (compute dtype): see axk_masked_attention in csrc/api.h.
+        `gate`: float32 rows (a view whose rows may be strided) of heads vdim gate logits, or None."""
+        self._elem(q, "attention q"); self._elem(out, "attention out")
+        self._i32(positions, "positions"); self._i32(seq_rows, "seq_rows"); self._i32(block_table, "block_table")
+        T = positions.numel()
+        if q.shape != (T, heads * maps * dim) or out.shape != (T, heads * vdim) or seq_rows.numel() != T \
+                or not q.is_contiguous() or not out.is_contiguous():
+            raise KernelError(f"masked_attention: q {tuple(q.shape)}, out {tuple(out.shape)} for {T} tokens")
+        self._check_heads_cache(cache, page_size, kv_heads * (maps * dim + vdim), "masked_attention")
+        if mask not in self.MASKS:
+            raise KernelError(f"masked_attention: mask '{mask}' is not known ({', '.join(self.MASKS)})")
+        gate_stride = 0
+        if gate is not None:
+            if gate.dtype != torch.float32 or gate.shape != (T, heads * vdim) or gate.stride(1) != 1:
+                raise KernelError(f"masked_attention: gate {tuple(gate.shape)} {gate.dtype} is not float32 [{T}, {heads * vdim}]")
+            gate_stride = gate.stride(0)
+        n_tiles = 0
+        if tiles is not None:
+            self._i32(tiles, "attention tiles")
+            n_tiles = tiles.shape[0]
+        self._check(self.lib.axk_masked_attention(
+            _ptr(q), _ptr(cache), _ptr(block_table), block_table.shape[-1], _ptr(positions), _ptr(seq_rows), _ptr(gate),
+            gate_stride, _ptr(out), T, heads, kv_heads, maps, dim, vdim, page_size, self.MASKS[mask], int(mask_size), float(scale),
+            float(softcap), float(lam), float(out_scale), float(eps), _ptr(tiles), n_tiles, _stream()))
+        return out
 
     def fill_i32(self, dst: torch.Tensor, value: int) -> None:
         self._i32(dst, "fill")

@@ -38,17 +38,23 @@ class DecoderModel:
             # a layer may have no feed-forward (its block then has to be one that takes none)
             ffn = build_part("feed_forward", layer.feed_forward, layer.prefix) if layer.feed_forward is not None else None
             self.blocks.append(build_block(layer.block, layer.norm, mixer, ffn, layer.prefix))
+        # rewrites of the residual stream that runs may enter through (they read the embedding's output)
+        self.entries = [build_part("stream", e) for e in spec.entries]
         self.final_norm = build_part("norm", spec.final_norm)
         self.head = build_part("head", spec.head)
         self.order = list(spec.order)
         for run in self.order:
             if not 0 <= run.layer < len(self.blocks):
                 raise ConfigError(f"the execution order names layer {run.layer}, the model has {len(self.blocks)}")
+            if run.enter is not None and not 0 <= run.enter < len(self.entries):
+                raise ConfigError(f"a run enters through entry {run.enter}, the model has {len(self.entries)}")
         self.cache_plan = self._plan_cache()
 
     # ------------------------------------------------------------------ declarations
     def tensors(self) -> List[TensorDecl]:
         out = list(self.embedding.tensors())
+        for e in self.entries:
+            out += e.tensors()
         for b in self.blocks:
             out += b.tensors()
         return out + self.final_norm.tensors() + self.head.tensors()
@@ -96,6 +102,8 @@ class DecoderModel:
     # ------------------------------------------------------------------ weights
     def load(self, store, rt) -> None:
         self.embedding.load(store, rt)
+        for e in self.entries:
+            e.load(store, rt)
         for b in self.blocks:
             b.load(store, rt)
         self.final_norm.load(store, rt)
@@ -108,7 +116,13 @@ class DecoderModel:
     # ------------------------------------------------------------------ the step
     def embed(self, ctx, out=None) -> torch.Tensor:
         """The residual stream before the first run: float32 [T, hidden] (into `out` if given)."""
-        return self.embedding.forward(ctx, out=out)
+        x = self.embedding.forward(ctx, out=out)
+        if self.entries:
+            # kept for the runs that enter through a rewrite of the stream; x itself moves on
+            x0 = ctx.ws.take(tuple(x.shape), torch.float32)
+            x0.copy_(x)
+            ctx.shared["embedding_output"] = x0
+        return x
 
     def forward(self, ctx) -> torch.Tensor:
         """The residual stream after every run: float32 [T, hidden]."""
@@ -122,8 +136,10 @@ class DecoderModel:
         for i in range(first, end):
             run, binding = self.order[i], self.cache_plan.bindings[i]
             block = self.blocks[run.layer]
+            if run.enter is not None:
+                self.entries[run.enter].forward(ctx, x, ctx.shared["embedding_output"])
             following = None
-            if i + 1 < end:
+            if i + 1 < end and self.order[i + 1].enter is None:     # a rewritten stream is normed by its own pass
                 after = self.blocks[self.order[i + 1].layer]
                 following = block.following_of(ctx, block.last_part(), after.first_norm(), x.shape[0])
             if normed is None and following is None:
@@ -135,7 +151,9 @@ class DecoderModel:
     def run_is_graph_safe(self, i: int) -> bool:
         """Whether run i's block and its parts are all fixed launch sequences (see Part.graph_safe)."""
         block = self.blocks[self.order[i].layer]
-        return all(getattr(p, "graph_safe", False) for p in (block, block.mixer, block.feed_forward) if p is not None)
+        entry = self.order[i].enter
+        parts = (block, block.mixer, block.feed_forward, None if entry is None else self.entries[entry])
+        return all(getattr(p, "graph_safe", False) for p in parts if p is not None)
 
     def ends_are_graph_safe(self) -> bool:
         """Whether what runs before the first run and behind the last (`embed`, `logits`) is a fixed

@@ -212,6 +212,15 @@ class FeedForward(Part):
         raise NotImplementedError
 
 
+class StreamEntry(Part):
+    """A rewrite of the residual stream between two runs: `forward(ctx, x, x0)` updates x [T, hidden]
+    (float32) in place from itself and x0, the embedding's output of this step (float32, not to be
+    changed).  A run of the execution order names one in its `enter`."""
+
+    def forward(self, ctx, x, x0) -> None:
+        raise NotImplementedError
+
+
 class Block(Part):
     """An arrangement: built from the layer's parts, not from a spec of its own.
 
@@ -258,7 +267,7 @@ class Block(Part):
 # --------------------------------------------------------------------------- registries
 
 _REGISTRIES: Dict[str, Dict[str, Any]] = {k: {} for k in
-                                          ("norm", "position", "mixer", "feed_forward", "block", "embedding", "head")}
+                                          ("norm", "position", "mixer", "feed_forward", "block", "embedding", "head", "stream")}
 
 
 def _register(kind: str, name: str, cls) -> None:
@@ -280,6 +289,7 @@ def register_feed_forward(name, cls): _register("feed_forward", name, cls)
 def register_block(name, cls): _register("block", name, cls)
 def register_embedding(name, cls): _register("embedding", name, cls)
 def register_head(name, cls): _register("head", name, cls)
+def register_stream(name, cls): _register("stream", name, cls)
 
 
 def build_part(kind: str, spec: PartSpec, prefix: str = "") -> Part:

@@ -62,6 +62,44 @@ class PreNormBlock(Block):
             self.feed_forward.forward(ctx, h, x)
 
 
+class ShortNamedPreNormBlock(PreNormBlock):
+    """The same arrangement for checkpoints that call the norms `norm1` and `norm2`; a layer may have no
+    feed-forward (it then has no second norm either)."""
+    norm1_name = "norm1"
+    norm2_name = "norm2"
+
+    def __init__(self, norm_factory, mixer, feed_forward, prefix):
+        Block.__init__(self, norm_factory, mixer, feed_forward, prefix)
+        self.norm1 = norm_factory(self.norm1_name)
+        self.norm2 = norm_factory(self.norm2_name) if feed_forward is not None else None
+
+    def parts(self):
+        return [p for p in (self.norm1, self.mixer, self.norm2, self.feed_forward) if p is not None]
+
+    def tensors(self) -> List[TensorDecl]:
+        return [d for p in self.parts() for d in p.tensors()]
+
+    def load(self, store, rt) -> None:
+        for part in self.parts():
+            part.load(store, rt)
+
+    def last_part(self):
+        return self.feed_forward if self.feed_forward is not None else self.mixer
+
+    def forward(self, ctx, binding: CacheBinding, x, normed=None, following=None) -> None:
+        if self.feed_forward is not None:
+            return super().forward(ctx, binding, x, normed, following)
+        h = normed
+        if h is None:
+            h = self.preceding_of(ctx, self.norm1, self.mixer, x)
+        if h is None:
+            h = self.norm1.forward(ctx, x)
+        if following is not None:
+            self.mixer.forward(ctx, binding, h, x, following)
+        else:
+            self.mixer.forward(ctx, binding, h, x)
+
+
 class SublayerNormBlock(Block):
     """x += mult * norm1(mixer(x)); x += mult * norm2(feed_forward(x)): the norms sit on the sublayers'
     outputs, the sublayers read the residual stream itself (rounded to the compute dtype for their
@@ -117,4 +155,5 @@ class SublayerNormBlock(Block):
 
 
 register_block("prenorm", PreNormBlock)
+register_block("prenorm_short_names", ShortNamedPreNormBlock)
 register_block("sublayer_norm", SublayerNormBlock)

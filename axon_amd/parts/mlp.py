@@ -59,7 +59,8 @@ register_feed_forward("swiglu_mlp", SwiGLUMLP)
 
 class DenseMLP(FeedForward):
     """down(act(up h)): a plain two-matrix feed-forward.  Parameters: `hidden_size`, `ff`,
-    `activation` ("gelu_tanh": 0.5 z (1 + tanh(sqrt(2 / pi) (z + 0.044715 z^3)))), `names` (scope "mlp.", up, down)."""
+    `activation` ("gelu_tanh": 0.5 z (1 + tanh(sqrt(2 / pi) (z + 0.044715 z^3))), or "gelu_erf":
+    0.5 z (1 + erf(z / sqrt 2))), `names` (scope "mlp.", up, down)."""
     graph_safe = True
     stores_output = True
 
@@ -67,8 +68,8 @@ class DenseMLP(FeedForward):
         super().__init__(params, prefix)
         self.hidden, self.ff = int(params["hidden_size"]), int(params["ff"])
         self.activation = params.get("activation", "gelu_tanh")
-        if self.activation != "gelu_tanh":
-            raise ConfigError(f"activation '{self.activation}' is not known (gelu_tanh)")
+        if self.activation not in ("gelu_tanh", "gelu_erf"):
+            raise ConfigError(f"activation '{self.activation}' is not known (gelu_tanh, gelu_erf)")
         names = params.get("names", {})
         base = prefix + names.get("scope", "mlp.")
         self.n = {k: base + names.get(k, k) for k in ("up", "down")}

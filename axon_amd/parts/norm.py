@@ -1,7 +1,9 @@
 """RMSNorm: rows of the 32-bit residual stream, normalised into the compute dtype.
 
 out = (x * 1/sqrt(mean(x^2) + eps)) * gain (src/model.rs:3888-3898).  Parameters: `size`,
-`eps`, `tensor` (the gain's name under the part's prefix).
+`eps`, `tensor` (the gain's name under the part's prefix), `offset` (default 0: the gain is
+offset + the stored vector, added once in 32-bit when the weights are loaded; 1 for checkpoints
+that store their gains around zero).
 """
 from __future__ import annotations
 
@@ -19,6 +21,7 @@ class RMSNorm(Norm):
         self.size = int(params["size"])
         self.eps = float(params["eps"])
         self.name = prefix + params.get("tensor", "weight")
+        self.offset = float(params.get("offset", 0.0))
         self.gain = None
 
     def tensors(self) -> List[TensorDecl]:
@@ -26,6 +29,8 @@ class RMSNorm(Norm):
 
     def load(self, store, rt) -> None:
         self.gain = store.vector(self.name)
+        if self.offset != 0.0:
+            self.gain = (self.gain.float() + self.offset).contiguous()      # kept 32-bit: 1 + w has more digits than w
 
     def forward(self, ctx, x, out=None, rows: Optional["torch.Tensor"] = None):
         """x: float32 [T, size]; `rows` picks rows of x (the wanted positions before the head)."""
