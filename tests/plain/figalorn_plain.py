@@ -162,12 +162,13 @@ def key_value_attention(h, W, p, m, eps):
         freqs, magnitude = base_frequencies(rot["dims"], rot["base"]), 1.0
     q, k = turn(q, pos, freqs, "halves", magnitude), turn(k, pos, freqs, "halves", magnitude)
     mask = window_mask(T, m["mask"]["size"])
-    cap = m["softcap"]
+    cap = m.get("softcap")
     heads = []
     for hd in range(H):
         g = hd // (H // G)
         s = q[:, hd] @ k[:, g].T * m["scale"]
-        s = cap * torch.tanh(s / cap)
+        if cap:
+            s = cap * torch.tanh(s / cap)
         heads.append(masked_softmax(s, mask) @ v[:, g])
     return torch.cat(heads, dim=-1) @ W[p + "o"].T
 
@@ -210,3 +211,15 @@ def forward(cfg, W, tokens, streams=None):
         if streams is not None:
             streams.append(x)
     return norm(x, W["final.norm"], eps) @ W["head"].T
+
+
+def greedy_generate(cfg, W, prompt, n_new):
+    """n_new tokens, each the largest logit after everything before it (ties to the larger id)."""
+    seq, out = list(prompt), []
+    for _ in range(n_new):
+        row = forward(cfg, W, seq)[-1]
+        best = float(row.max())
+        tok = max(i for i in range(row.numel()) if float(row[i]) == best)
+        seq.append(tok)
+        out.append(tok)
+    return out
