@@ -26,7 +26,7 @@ __device__ inline int first_seen(int pos, int mask_kind, int mask_size) {
   return 0;
 }
 
-// One block per token, a wave a unit (one map of one head) at a time.  proj [T, stride] float32 holds
+// One block per token (or several side by side, each with its share of the units), a wave a unit (one map of one head) at a time.  proj [T, stride] float32 holds
 // the projections' results: n_q units of `dim` from q_at, n_k units from k_at, and v_width values from
 // v_at (v_at may equal k_at: the values are the keys as projected).  Units are RMS-normed with a gain
 // shared by all units (if given), their first rot dims rotated by the step's table [T, rot / 2, 2]
@@ -52,7 +52,7 @@ heads_prepare_kernel(const float* __restrict__ proj, long stride, int q_at, int 
     in_page = pos % page_size;
   }
   const int n_units = n_q + (write_kv ? n_k : 0);
-  for (int u = wave; u < n_units; u += 4) {
+  for (int u = blockIdx.y * 4 + wave; u < n_units; u += 4 * gridDim.y) {
     const bool is_q = u < n_q;
     const float* src = row + (is_q ? q_at + u * dim : k_at + (u - n_q) * dim);
     elem_t* dst = is_q ? q_out + ((long)t * n_q + u) * dim : page_base + (long)in_page * kw + (long)(u - n_q) * dim;
@@ -83,7 +83,7 @@ heads_prepare_kernel(const float* __restrict__ proj, long stride, int q_at, int 
   }
   if (!write_kv) return;
   elem_t* by_dim = page_base + (long)page_size * kw + in_page;
-  for (int i = threadIdx.x; i < v_width; i += 256) by_dim[(long)i * page_size] = from_float(row[v_at + i]);
+  for (int i = blockIdx.y * 256 + threadIdx.x; i < v_width; i += 256 * gridDim.y) by_dim[(long)i * page_size] = from_float(row[v_at + i]);
 }
 
 // One wave per (token, head), four waves a block; any sizes, both builds.  For each map: positions
@@ -194,18 +194,175 @@ __device__ inline ma_bf16x8 ma_frag(uint4 v) { return __builtin_bit_cast(ma_bf16
 //   positions of its column; the four lanes of a column meet by lane permutation), the running
 //   (m, l) and O^T rescaled, then
 //   O^T [dim, column] += V^T [dim, position] P^T             (positions in two chunks of 32),
-// with K rows and the rows of V^T straight from the page into the first operand (16 or 8 bytes a lane)
-// and the rounded weights, as they lie in the accumulators, as the second.  Both maps of a
-// differential head run side by side over one load of the values; the combination, the norm and the
-// gate happen in registers before the store.  DT: tiles of 16 value dims at most; KC: chunks of 32 key
-// dims at most.  Pages hold a multiple of 64 positions, dim is a multiple of 8, vdim of 16.
+// with K rows and the rows of V^T as the first operand (16 or 8 bytes a lane) and the rounded
+// weights, as they lie in the accumulators, as the second.  Both maps of a differential head run
+// side by side over one load of the values; the combination, the norm and the gate happen in
+// registers before the store.  DT: tiles of 16 value dims at most; KC: chunks of 32 key dims at
+// most.  Pages hold a multiple of 64 positions, dim is a multiple of 8, vdim of 16.
+template <int MAPS, int DT>
+struct MaState {
+  ma_f32x4 acc[MAPS][DT];
+  float m[MAPS], l[MAPS];
+  __device__ inline void clear() {
+#pragma unroll
+    for (int mp = 0; mp < MAPS; ++mp) {
+      m[mp] = -INFINITY;
+      l[mp] = 0.0f;
+#pragma unroll
+      for (int i = 0; i < DT; ++i) acc[mp][i] = ma_f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+    }
+  }
+};
+
+// One block of 64 positions from p0 for a wave's columns.  kbase: the block's first key row of the
+// wave's key/value head, rows kstride apart (a map's keys mp * dim further); vbase: its first value
+// row, rows vstride apart, the block's positions side by side; both already moved to the lane's
+// slice (8 g, 4 g).  qfrag(mp, c): the lane's query operand of map mp, chunk c.
+template <int MAPS, int DT, int KC, class QF>
+__device__ inline void ma_block(MaState<MAPS, DT>& st, const bf16_t* kbase, long kstride, const bf16_t* vbase, long vstride,
+                                QF qfrag, int p0, int my_lo, int my_pos, int dim, int dt_n, float scale, float softcap, int j,
+                                int g) {
+  const int kc = (dim + 31) / 32;
+  uint4 pf[MAPS][2];
+  float fold[MAPS];
+#pragma unroll
+  for (int mp = 0; mp < MAPS; ++mp) {
+    ma_f32x4 s[4];
+#pragma unroll
+    for (int pt = 0; pt < 4; ++pt) {
+      s[pt] = ma_f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+      const bf16_t* krow = kbase + (long)(16 * pt + j) * kstride + mp * dim;
+      uint4 kf[KC];
+#pragma unroll
+      for (int c = 0; c < KC; ++c)
+        kf[c] = (c < kc && 32 * c + 8 * g < dim) ? *reinterpret_cast<const uint4*>(krow + 32 * c) : make_uint4(0u, 0u, 0u, 0u);
+#pragma unroll
+      for (int c = 0; c < KC; ++c)
+        if (c < kc) s[pt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ma_frag(kf[c]), ma_frag(qfrag(mp, c)), s[pt], 0, 0, 0);
+    }
+    float mx = -INFINITY;
+#pragma unroll
+    for (int pt = 0; pt < 4; ++pt)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int p = p0 + 16 * pt + 4 * g + i;
+        float v = s[pt][i] * scale;
+        if (softcap > 0.0f) v = softcap * tanhf(v / softcap);
+        v = (p >= my_lo && p <= my_pos) ? v : -INFINITY;
+        s[pt][i] = v;
+        mx = fmaxf(mx, v);
+      }
+    mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+    const float m_new = fmaxf(st.m[mp], mx);
+    const float m_safe = m_new == -INFINITY ? 0.0f : m_new;      // a column that has seen nothing yet
+    fold[mp] = expf(st.m[mp] - m_safe);
+    float sum = 0.0f;
+#pragma unroll
+    for (int pt = 0; pt < 4; ++pt)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const float w = expf(s[pt][i] - m_safe);        // 0 where the position is not seen
+        s[pt][i] = w;
+        sum += w;
+      }
+    sum += __shfl_xor(sum, 16, 64);
+    sum += __shfl_xor(sum, 32, 64);
+    st.l[mp] = fmaf(st.l[mp], fold[mp], sum);
+    st.m[mp] = m_new;
+#pragma unroll
+    for (int c = 0; c < 2; ++c)
+      pf[mp][c] = make_uint4(pack2_bf16(s[2 * c][0], s[2 * c][1]), pack2_bf16(s[2 * c][2], s[2 * c][3]),
+                             pack2_bf16(s[2 * c + 1][0], s[2 * c + 1][1]), pack2_bf16(s[2 * c + 1][2], s[2 * c + 1][3]));
+  }
+  constexpr int VB = DT < 4 ? DT : 4;                         // tiles of 16 dims whose rows are asked for together
+#pragma unroll
+  for (int d0 = 0; d0 < DT; d0 += VB) {
+    uint2 v[VB][4];
+#pragma unroll
+    for (int e = 0; e < VB; ++e) {
+      if (d0 + e < dt_n) {
+        const bf16_t* vrow = vbase + (long)(16 * (d0 + e) + j) * vstride;
+#pragma unroll
+        for (int c = 0; c < 2; ++c) {
+          v[e][2 * c] = *reinterpret_cast<const uint2*>(vrow + 32 * c);
+          v[e][2 * c + 1] = *reinterpret_cast<const uint2*>(vrow + 32 * c + 16);
+        }
+      }
+    }
+#pragma unroll
+    for (int e = 0; e < VB; ++e) {
+      if (d0 + e < dt_n) {
+#pragma unroll
+        for (int mp = 0; mp < MAPS; ++mp) {
+          st.acc[mp][d0 + e] *= fold[mp];
+#pragma unroll
+          for (int c = 0; c < 2; ++c)
+            st.acc[mp][d0 + e] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                ma_frag(make_uint4(v[e][2 * c].x, v[e][2 * c].y, v[e][2 * c + 1].x, v[e][2 * c + 1].y)), ma_frag(pf[mp][c]),
+                st.acc[mp][d0 + e], 0, 0, 0);
+        }
+      }
+    }
+  }
+}
+
+// A column's outputs (dims 16 dt + 4 g + i in the four lanes j, j + 16, j + 32, j + 48): the maps
+// combined, normed, gated and stored.
+template <int MAPS, int DT>
+__device__ inline void ma_finish(MaState<MAPS, DT>& st, bool my_col, int my_tok, int my_head, int heads, int vdim, int dt_n,
+                                 const float* __restrict__ gate, long gate_stride, bf16_t* __restrict__ out, float lambda,
+                                 float out_scale, float eps, int g) {
+  const float inv0 = 1.0f / st.l[0];
+  float ss = 0.0f;
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt)
+    if (dt < dt_n) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        float o = st.acc[0][dt][i] * inv0;
+        if (MAPS == 2) {
+          o = o - lambda * (st.acc[MAPS - 1][dt][i] * (1.0f / st.l[MAPS - 1]));
+          ss = fmaf(o, o, ss);
+        }
+        st.acc[0][dt][i] = o;
+      }
+    }
+  float norm = 1.0f;
+  if (MAPS == 2) {
+    ss += __shfl_xor(ss, 16, 64);
+    ss += __shfl_xor(ss, 32, 64);
+    norm = (1.0f / sqrtf(ss / (float)vdim + eps));
+  }
+  if (!my_col) return;
+  bf16_t* dst = out + ((long)my_tok * heads + my_head) * vdim + 4 * g;
+  const float* gsrc = gate ? gate + (long)my_tok * gate_stride + (long)my_head * vdim + 4 * g : nullptr;
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt)
+    if (dt < dt_n) {
+      float o[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        o[i] = st.acc[0][dt][i];
+        if (MAPS == 2) o[i] = (o[i] * norm) * out_scale;
+        if (gsrc) o[i] *= 1.0f / (1.0f + expf(-gsrc[16 * dt + i]));
+      }
+      *reinterpret_cast<uint2*>(dst + 16 * dt) = make_uint2(pack2_bf16(o[0], o[1]), pack2_bf16(o[2], o[3]));
+    }
+}
+
+// Keys, values and queries straight from memory, a wave a block.  grid (tiles, heads, chunks): with
+// `partial` (steps of few single tokens under a window or in chunks) the wave of chunk c takes the
+// c-th block of 64 positions of its token alone and leaves (o, m, l) of every column and map,
+// unscaled, for the kernel that folds a token's blocks in ascending order; without, it walks them all.
 template <int MAPS, int DT, int KC>
 __global__ void __launch_bounds__(64)
 masked_attention_mfma_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ cache, const int32_t* __restrict__ block_table,
                              int table_stride, const int32_t* __restrict__ positions, const int32_t* __restrict__ seq_rows,
                              const float* __restrict__ gate, long gate_stride, bf16_t* __restrict__ out,
                              const int32_t* __restrict__ tiles, int heads, int kv_heads, int dim, int vdim, int page_size,
-                             int mask_kind, int mask_size, float scale, float softcap, float lambda, float out_scale, float eps) {
+                             int mask_kind, int mask_size, float scale, float softcap, float lambda, float out_scale, float eps,
+                             float* __restrict__ partial, int n_chunks) {
   constexpr int QMAP = KC * 32, QROW = MAPS * QMAP + 8;      // rows 16 bytes longer than their chunks: 16 rows, 16 banks apart
   __shared__ __align__(16) bf16_t qs[16 * QROW];
   const int lane = threadIdx.x, j = lane & 15, g = lane >> 4;
@@ -242,156 +399,218 @@ masked_attention_mfma_kernel(const bf16_t* __restrict__ q, const bf16_t* __restr
   const int pos_first = positions[t0], pos_last = pos_first + n - 1;
   const int lo_first = first_seen(pos_first, mask_kind, mask_size);
   const int32_t* pages = block_table + (long)seq_rows[t0] * table_stride;
-  const int kw = kv_heads * MAPS * dim, kc = (dim + 31) / 32, dt_n = vdim / 16;
+  const int kw = kv_heads * MAPS * dim, dt_n = vdim / 16;
   const long page_elems = (long)page_size * (kw + kv_heads * vdim);
   const bf16_t* qlane = qs + j * QROW + 8 * g;
-  ma_f32x4 acc[MAPS][DT];
-  float m[MAPS], l[MAPS];
-#pragma unroll
-  for (int mp = 0; mp < MAPS; ++mp) {
-    m[mp] = -INFINITY;
-    l[mp] = 0.0f;
-#pragma unroll
-    for (int i = 0; i < DT; ++i) acc[mp][i] = ma_f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+  auto qfrag = [&](int mp, int c) { return *reinterpret_cast<const uint4*>(qlane + mp * QMAP + 32 * c); };
+  MaState<MAPS, DT> st;
+  st.clear();
+  const bool split = partial != nullptr && n == 1;
+  if (!split && blockIdx.z > 0) return;
+  const int b_first = split ? lo_first / 64 + (int)blockIdx.z : lo_first / 64;
+  const int b_last = split ? min(b_first, pos_last / 64) : pos_last / 64;
+  for (int b = b_first; b <= b_last; ++b) {
+    const int p0 = b * 64, in0 = p0 % page_size;
+    const bf16_t* page = cache + (long)pages[p0 / page_size] * page_elems;
+    ma_block<MAPS, DT, KC>(st, page + (long)in0 * kw + (long)gk * MAPS * dim + 8 * g, kw,
+                           page + (long)page_size * kw + (long)gk * vdim * page_size + in0 + 4 * g, page_size, qfrag, p0, my_lo,
+                           my_pos, dim, dt_n, scale, softcap, j, g);
   }
+  if (split) {
+    if (!my_col) return;
+#pragma unroll
+    for (int mp = 0; mp < MAPS; ++mp) {
+      float* dst = partial + ((((long)my_tok * heads + my_head) * n_chunks + blockIdx.z) * MAPS + mp) * (vdim + 2);
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt)
+        if (dt < dt_n) {
+#pragma unroll
+          for (int i = 0; i < 4; ++i) dst[16 * dt + 4 * g + i] = st.acc[mp][dt][i];
+        }
+      if (g == 0) {
+        dst[vdim] = st.m[mp];
+        dst[vdim + 1] = st.l[mp];
+      }
+    }
+    return;
+  }
+  ma_finish<MAPS, DT>(st, my_col, my_tok, my_head, heads, vdim, dt_n, gate, gate_stride, out, lambda, out_scale, eps, g);
+}
+
+// The blocks of a single token's (head, map) folded in ascending order, a_mp = sum_c e^(m_c - M) o_c /
+// sum_c e^(m_c - M) l_c (M the largest m_c; a block that saw nothing has l = 0 and weighs nothing), then
+// the maps combined, normed, gated and stored.  One wave per (tile, head); tiles of several tokens were
+// finished by the attention kernel itself.
+template <int MAPS>
+__global__ void __launch_bounds__(64)
+masked_attention_fold_kernel(const float* __restrict__ partial, int n_chunks, const int32_t* __restrict__ tiles,
+                             const float* __restrict__ gate, long gate_stride, bf16_t* __restrict__ out, int heads, int vdim,
+                             float lambda, float out_scale, float eps) {
+  const int t = tiles ? tiles[2 * blockIdx.x] : (int)blockIdx.x, n = tiles ? tiles[2 * blockIdx.x + 1] : 1;
+  if (n != 1) return;
+  const int h = blockIdx.y, lane = threadIdx.x;
+  float o[MA_OWN];
+#pragma unroll
+  for (int i = 0; i < MA_OWN; ++i) o[i] = 0.0f;
+  for (int mp = 0; mp < MAPS; ++mp) {
+    const float* src = partial + (((long)t * heads + h) * n_chunks * MAPS + mp) * (vdim + 2);
+    const long step = (long)MAPS * (vdim + 2);
+    float M = -INFINITY;
+    for (int c = 0; c < n_chunks; ++c)
+      if (src[c * step + vdim + 1] > 0.0f) M = fmaxf(M, src[c * step + vdim]);
+    float L = 0.0f, acc[MA_OWN];
+#pragma unroll
+    for (int i = 0; i < MA_OWN; ++i) acc[i] = 0.0f;
+    for (int c = 0; c < n_chunks; ++c) {
+      const float lc = src[c * step + vdim + 1];
+      if (!(lc > 0.0f)) continue;
+      const float w = expf(src[c * step + vdim] - M);
+      L = fmaf(w, lc, L);
+#pragma unroll
+      for (int i = 0; i < MA_OWN; ++i) {
+        const int d = lane + 64 * i;
+        if (d < vdim) acc[i] = fmaf(w, src[c * step + d], acc[i]);
+      }
+    }
+    const float inv = 1.0f / L;
+#pragma unroll
+    for (int i = 0; i < MA_OWN; ++i) o[i] = mp == 0 ? acc[i] * inv : o[i] - lambda * (acc[i] * inv);
+  }
+  if (MAPS > 1) {
+    float ss = 0.0f;
+#pragma unroll
+    for (int i = 0; i < MA_OWN; ++i) ss = fmaf(o[i], o[i], ss);
+    const float inv = 1.0f / sqrtf(wave_sum(ss) / (float)vdim + eps);
+#pragma unroll
+    for (int i = 0; i < MA_OWN; ++i) o[i] = (o[i] * inv) * out_scale;
+  }
+  bf16_t* dst = out + ((long)t * heads + h) * vdim;
+#pragma unroll
+  for (int i = 0; i < MA_OWN; ++i) {
+    const int d = lane + 64 * i;
+    if (d >= vdim) continue;
+    float v = o[i];
+    if (gate != nullptr) v *= 1.0f / (1.0f + expf(-gate[(long)t * gate_stride + (long)h * vdim + d]));
+    dst[d] = from_float(v);
+  }
+}
+
+// Steps with portions of prompts: four waves a block, the four query heads of one key/value head (or as
+// many as the group has) on the same tile of tokens.  A block of 64 positions of that head's keys and
+// values goes through LDS once for all four (rows 16 bytes longer than their data, against bank
+// conflicts), queries wait in registers as operands.  A tile of one token is its first wave's alone
+// (up to sixteen heads as columns).
+#define MAS_WAVES 4
+template <int MAPS, int DT, int KC>
+__global__ void __launch_bounds__(MAS_WAVES * 64)
+masked_attention_staged_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ cache,
+                               const int32_t* __restrict__ block_table, int table_stride, const int32_t* __restrict__ positions,
+                               const int32_t* __restrict__ seq_rows, const float* __restrict__ gate, long gate_stride,
+                               bf16_t* __restrict__ out, const int32_t* __restrict__ tiles, int heads, int kv_heads, int dim,
+                               int vdim, int page_size, int mask_kind, int mask_size, float scale, float softcap, float lambda,
+                               float out_scale, float eps) {
+  extern __shared__ __align__(16) bf16_t stage[];       // keys [64][MAPS dim + 8], then values [vdim][64 + 8]
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, j = lane & 15, g = lane >> 4;
+  const int grp = heads / kv_heads, hb_n = (grp + MAS_WAVES - 1) / MAS_WAVES;
+  const int t0 = tiles[2 * blockIdx.x], n = tiles[2 * blockIdx.x + 1];
+  const int gk = blockIdx.y / hb_n, hb = blockIdx.y % hb_n;
+  int h0, ncols;
+  bool active;
+  if (n == 1) {
+    const int hc = grp < 16 ? grp : 16, per_kv = (grp + hc - 1) / hc;
+    if (hb >= per_kv) return;                           // the whole block: nothing waits for it
+    h0 = gk * grp + hb * hc;
+    ncols = min(hc, grp - hb * hc);
+    active = wave == 0;
+  } else {
+    h0 = gk * grp + hb * MAS_WAVES + wave;
+    ncols = n;
+    active = hb * MAS_WAVES + wave < grp;
+  }
+  const int my_tok = n == 1 ? t0 : t0 + j, my_head = n == 1 ? h0 + j : h0;
+  const bool my_col = active && j < ncols;
+  const int qw = MAPS * dim;
+  uint4 qf[MAPS][KC];
+#pragma unroll
+  for (int mp = 0; mp < MAPS; ++mp)
+#pragma unroll
+    for (int c = 0; c < KC; ++c)
+      qf[mp][c] = (my_col && 32 * c + 8 * g < dim)
+                      ? *reinterpret_cast<const uint4*>(q + ((long)my_tok * heads + my_head) * qw + mp * dim + 32 * c + 8 * g)
+                      : make_uint4(0u, 0u, 0u, 0u);
+  auto qfrag = [&](int mp, int c) { return qf[mp][c]; };
+  const int my_pos = my_col ? positions[my_tok] : -1;
+  const int my_lo = my_col ? first_seen(my_pos, mask_kind, mask_size) : 0;
+  const int pos_first = positions[t0], pos_last = pos_first + n - 1;
+  const int lo_first = first_seen(pos_first, mask_kind, mask_size);
+  const int32_t* pages = block_table + (long)seq_rows[t0] * table_stride;
+  const int kw = kv_heads * MAPS * dim, dt_n = vdim / 16;
+  const long page_elems = (long)page_size * (kw + kv_heads * vdim);
+  const int krow = qw + 8, vrow = 64 + 8, k_pieces = qw / 8;
+  bf16_t* ks = stage;
+  bf16_t* vs = stage + 64 * krow;
+  MaState<MAPS, DT> st;
+  st.clear();
   for (int b = lo_first / 64; b <= pos_last / 64; ++b) {
     const int p0 = b * 64, in0 = p0 % page_size;
     const bf16_t* page = cache + (long)pages[p0 / page_size] * page_elems;
-    const bf16_t* kbase = page + (long)in0 * kw + (long)gk * MAPS * dim + 8 * g;
-    const bf16_t* vbase = page + (long)page_size * kw + (long)gk * vdim * page_size + in0 + 4 * g;
-    uint4 pf[MAPS][2];
-    float fold[MAPS];
-#pragma unroll
-    for (int mp = 0; mp < MAPS; ++mp) {
-      ma_f32x4 s[4];
-#pragma unroll
-      for (int pt = 0; pt < 4; ++pt) {
-        s[pt] = ma_f32x4{0.0f, 0.0f, 0.0f, 0.0f};
-        const bf16_t* krow = kbase + (long)(16 * pt + j) * kw + mp * dim;
-        uint4 kf[KC];
-#pragma unroll
-        for (int c = 0; c < KC; ++c)
-          kf[c] = (c < kc && 32 * c + 8 * g < dim) ? *reinterpret_cast<const uint4*>(krow + 32 * c) : make_uint4(0u, 0u, 0u, 0u);
-#pragma unroll
-        for (int c = 0; c < KC; ++c)
-          if (c < kc)
-            s[pt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
-                ma_frag(kf[c]), ma_frag(*reinterpret_cast<const uint4*>(qlane + mp * QMAP + 32 * c)), s[pt], 0, 0, 0);
-      }
-      float mx = -INFINITY;
-#pragma unroll
-      for (int pt = 0; pt < 4; ++pt)
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const int p = p0 + 16 * pt + 4 * g + i;
-          float v = s[pt][i] * scale;
-          if (softcap > 0.0f) v = softcap * tanhf(v / softcap);
-          v = (p >= my_lo && p <= my_pos) ? v : -INFINITY;
-          s[pt][i] = v;
-          mx = fmaxf(mx, v);
-        }
-      mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-      mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-      const float m_new = fmaxf(m[mp], mx);
-      const float m_safe = m_new == -INFINITY ? 0.0f : m_new;      // a column that has seen nothing yet
-      fold[mp] = expf(m[mp] - m_safe);
-      float sum = 0.0f;
-#pragma unroll
-      for (int pt = 0; pt < 4; ++pt)
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const float w = expf(s[pt][i] - m_safe);        // 0 where the position is not seen
-          s[pt][i] = w;
-          sum += w;
-        }
-      sum += __shfl_xor(sum, 16, 64);
-      sum += __shfl_xor(sum, 32, 64);
-      l[mp] = fmaf(l[mp], fold[mp], sum);
-      m[mp] = m_new;
-#pragma unroll
-      for (int c = 0; c < 2; ++c)
-        pf[mp][c] = make_uint4(pack2_bf16(s[2 * c][0], s[2 * c][1]), pack2_bf16(s[2 * c][2], s[2 * c][3]),
-                               pack2_bf16(s[2 * c + 1][0], s[2 * c + 1][1]), pack2_bf16(s[2 * c + 1][2], s[2 * c + 1][3]));
+    const bf16_t* ksrc = page + (long)in0 * kw + (long)gk * qw;
+    const bf16_t* vsrc = page + (long)page_size * kw + (long)gk * vdim * page_size + in0;
+    __syncthreads();                                    // the block before has been read
+    for (int idx = threadIdx.x; idx < 64 * k_pieces; idx += MAS_WAVES * 64) {
+      const int r = idx / k_pieces, piece = idx % k_pieces;
+      *reinterpret_cast<uint4*>(ks + r * krow + 8 * piece) = *reinterpret_cast<const uint4*>(ksrc + (long)r * kw + 8 * piece);
     }
-    constexpr int VB = DT < 4 ? DT : 4;                         // tiles of 16 dims whose rows are asked for together
-#pragma unroll
-    for (int d0 = 0; d0 < DT; d0 += VB) {
-      uint2 v[VB][4];
-#pragma unroll
-      for (int e = 0; e < VB; ++e) {
-        if (d0 + e < dt_n) {
-          const bf16_t* vrow = vbase + (long)(16 * (d0 + e) + j) * page_size;
-#pragma unroll
-          for (int c = 0; c < 2; ++c) {
-            v[e][2 * c] = *reinterpret_cast<const uint2*>(vrow + 32 * c);
-            v[e][2 * c + 1] = *reinterpret_cast<const uint2*>(vrow + 32 * c + 16);
-          }
-        }
-      }
-#pragma unroll
-      for (int e = 0; e < VB; ++e) {
-        if (d0 + e < dt_n) {
-#pragma unroll
-          for (int mp = 0; mp < MAPS; ++mp) {
-            acc[mp][d0 + e] *= fold[mp];
-#pragma unroll
-            for (int c = 0; c < 2; ++c)
-              acc[mp][d0 + e] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
-                  ma_frag(make_uint4(v[e][2 * c].x, v[e][2 * c].y, v[e][2 * c + 1].x, v[e][2 * c + 1].y)), ma_frag(pf[mp][c]),
-                  acc[mp][d0 + e], 0, 0, 0);
-          }
-        }
-      }
+    for (int idx = threadIdx.x; idx < vdim * 8; idx += MAS_WAVES * 64) {
+      const int r = idx >> 3, piece = idx & 7;
+      *reinterpret_cast<uint4*>(vs + r * vrow + 8 * piece) = *reinterpret_cast<const uint4*>(vsrc + (long)r * page_size + 8 * piece);
     }
+    __syncthreads();
+    if (active)
+      ma_block<MAPS, DT, KC>(st, ks + 8 * g, krow, vs + 4 * g, vrow, qfrag, p0, my_lo, my_pos, dim, dt_n, scale, softcap, j, g);
   }
-  // a column's outputs: dims 16 dt + 4 g + i in the four lanes j, j + 16, j + 32, j + 48
-  const float inv0 = 1.0f / l[0];
-  float ss = 0.0f;
-#pragma unroll
-  for (int dt = 0; dt < DT; ++dt)
-    if (dt < dt_n) {
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        float o = acc[0][dt][i] * inv0;
-        if (MAPS == 2) {
-          o = o - lambda * (acc[MAPS - 1][dt][i] * (1.0f / l[MAPS - 1]));
-          ss = fmaf(o, o, ss);
-        }
-        acc[0][dt][i] = o;
-      }
-    }
-  float norm = 1.0f;
-  if (MAPS == 2) {
-    ss += __shfl_xor(ss, 16, 64);
-    ss += __shfl_xor(ss, 32, 64);
-    norm = (1.0f / sqrtf(ss / (float)vdim + eps));
-  }
-  if (!my_col) return;
-  bf16_t* dst = out + ((long)my_tok * heads + my_head) * vdim + 4 * g;
-  const float* gsrc = gate ? gate + (long)my_tok * gate_stride + (long)my_head * vdim + 4 * g : nullptr;
-#pragma unroll
-  for (int dt = 0; dt < DT; ++dt)
-    if (dt < dt_n) {
-      float o[4];
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        o[i] = acc[0][dt][i];
-        if (MAPS == 2) o[i] = (o[i] * norm) * out_scale;
-        if (gsrc) o[i] *= 1.0f / (1.0f + expf(-gsrc[16 * dt + i]));
-      }
-      *reinterpret_cast<uint2*>(dst + 16 * dt) = make_uint2(pack2_bf16(o[0], o[1]), pack2_bf16(o[2], o[3]));
-    }
+  if (active)
+    ma_finish<MAPS, DT>(st, my_col, my_tok, my_head, heads, vdim, dt_n, gate, gate_stride, out, lambda, out_scale, eps, g);
+}
+
+// Blocks of positions a single token can touch under its mask (0: no bound).
+static int masked_chunks(int mask_kind, int mask_size) {
+  return mask_kind == MASK_CAUSAL ? 0 : (mask_size + 62) / 64 + 1;
 }
 
 template <int MAPS, int DT, int KC>
-static void launch_masked_mfma(const void* q, const void* cache, const int32_t* block_table, int table_stride,
-                               const int32_t* positions, const int32_t* seq_rows, const float* gate, long gate_stride, void* out,
-                               const int32_t* tiles, int n_tiles, int heads, int kv_heads, int dim, int vdim, int page_size,
-                               int mask_kind, int mask_size, float scale, float softcap, float lambda, float out_scale, float eps,
-                               hipStream_t stream) {
-  masked_attention_mfma_kernel<MAPS, DT, KC><<<dim3(n_tiles, heads), 64, 0, stream>>>(
+static int launch_masked_mfma(const void* q, const void* cache, const int32_t* block_table, int table_stride,
+                              const int32_t* positions, const int32_t* seq_rows, const float* gate, long gate_stride, void* out,
+                              const int32_t* tiles, int n_tiles, int heads, int kv_heads, int dim, int vdim, int page_size,
+                              int mask_kind, int mask_size, float scale, float softcap, float lambda, float out_scale, float eps,
+                              float* partial, hipStream_t stream) {
+  const int grp = heads / kv_heads;
+  const size_t lds = ((size_t)64 * (MAPS * dim + 8) + (size_t)vdim * (64 + 8)) * sizeof(bf16_t);
+  if (tiles != nullptr && partial == nullptr && KC <= 4 && lds <= 64 * 1024) {
+    static bool configured = false;
+    if (!configured && lds > 48 * 1024) {
+      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&masked_attention_staged_kernel<MAPS, DT, KC>),
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, 64 * 1024);
+      if (e != hipSuccess) {
+        axk_set_error("masked_attention: cannot reserve %d bytes of LDS: %s", 64 * 1024, hipGetErrorString(e));
+        return -2;
+      }
+      configured = true;
+    }
+    masked_attention_staged_kernel<MAPS, DT, KC>
+        <<<dim3(n_tiles, kv_heads * ((grp + MAS_WAVES - 1) / MAS_WAVES)), MAS_WAVES * 64, lds, stream>>>(
+            (const bf16_t*)q, (const bf16_t*)cache, block_table, table_stride, positions, seq_rows, gate, gate_stride,
+            (bf16_t*)out, tiles, heads, kv_heads, dim, vdim, page_size, mask_kind, mask_size, scale, softcap, lambda, out_scale, eps);
+    return 0;
+  }
+  const int n_chunks = partial ? masked_chunks(mask_kind, mask_size) : 1;
+  masked_attention_mfma_kernel<MAPS, DT, KC><<<dim3(n_tiles, heads, n_chunks), 64, 0, stream>>>(
       (const bf16_t*)q, (const bf16_t*)cache, block_table, table_stride, positions, seq_rows, gate, gate_stride, (bf16_t*)out, tiles,
-      heads, kv_heads, dim, vdim, page_size, mask_kind, mask_size, scale, softcap, lambda, out_scale, eps);
+      heads, kv_heads, dim, vdim, page_size, mask_kind, mask_size, scale, softcap, lambda, out_scale, eps, partial, n_chunks);
+  if (partial)
+    masked_attention_fold_kernel<MAPS><<<dim3(n_tiles, heads), 64, 0, stream>>>(partial, n_chunks, tiles, gate, gate_stride,
+                                                                              (bf16_t*)out, heads, vdim, lambda, out_scale, eps);
+  return 0;
 }
 #endif
 
@@ -409,7 +628,9 @@ extern "C" int axk_heads_prepare(const float* proj, long stride, int q_at, int n
   AXK_REQUIRE(q_at >= 0 && k_at >= 0 && v_at >= 0 && q_at + (long)n_q * dim <= stride && k_at + (long)n_k * dim <= stride &&
               v_at + (long)v_width <= stride, "heads_prepare: the parts do not fit rows of %ld", stride);
   if (n_tokens == 0) return 0;
-  heads_prepare_kernel<<<n_tokens, 256, 0, (hipStream_t)stream>>>(
+  // few tokens: a token's units side by side in several blocks
+  const int per_token = n_tokens >= 1024 ? 1 : min((n_q + n_k + 3) / 4, 16);
+  heads_prepare_kernel<<<dim3(n_tokens, per_token), 256, 0, (hipStream_t)stream>>>(
       proj, stride, q_at, n_q, k_at, n_k, v_at, v_width, dim, q_gain, q_gain_is_f32, k_gain, k_gain_is_f32, eps, rot, neighbours,
       magnitude, table, positions, seq_rows, block_table, table_stride, (elem_t*)cache, page_size, (elem_t*)q_out, write_kv);
   AXK_LAUNCH_CHECK("heads_prepare");
@@ -425,11 +646,27 @@ extern "C" int axk_masked_attention_uses_mfma(int heads, int kv_heads, int maps,
 #endif
 }
 
+// Steps of few tokens under a window or in chunks: the blocks of 64 positions of a single token run side
+// by side and a second launch folds them; the floats of the workspace that takes (0: a wave walks its
+// token's blocks itself).
+extern "C" long axk_masked_attention_workspace(int n_tokens, int heads, int kv_heads, int maps, int dim, int vdim, int page_size,
+                                               int mask_kind, int mask_size) {
+#if AXON_BF16
+  if (!axk_masked_attention_uses_mfma(heads, kv_heads, maps, dim, vdim, page_size)) return 0;
+  const int chunks = masked_chunks(mask_kind, mask_size);
+  if (chunks < 3 || (long)n_tokens * kv_heads >= 512) return 0;
+  return (long)n_tokens * heads * chunks * maps * (vdim + 2);
+#else
+  return 0;
+#endif
+}
+
 extern "C" int axk_masked_attention(const void* q, const void* cache, const int32_t* block_table, int table_stride,
                                     const int32_t* positions, const int32_t* seq_rows, const float* gate, long gate_stride,
                                     void* out, int n_tokens, int heads, int kv_heads, int maps, int dim, int vdim, int page_size,
                                     int mask_kind, int mask_size, float scale, float softcap, float lambda, float out_scale,
-                                    float eps, const int32_t* tiles, int n_tiles, void* stream) {
+                                    float eps, const int32_t* tiles, int n_tiles, float* partial, long partial_floats,
+                                    void* stream) {
   AXK_REQUIRE(n_tokens >= 0 && heads > 0 && kv_heads > 0 && heads % kv_heads == 0 && dim > 0 && vdim > 0 && page_size > 0,
               "masked_attention: bad sizes T=%d heads=%d kv heads=%d dim=%d vdim=%d page=%d", n_tokens, heads, kv_heads, dim, vdim,
               page_size);
@@ -445,16 +682,22 @@ extern "C" int axk_masked_attention(const void* q, const void* cache, const int3
     AXK_REQUIRE(tiles == nullptr || n_tiles > 0, "masked_attention: a list of %d tiles", n_tiles);
     const int nt = tiles ? n_tiles : n_tokens;
     const int size = dim > vdim ? dim : vdim;
+    const long need = axk_masked_attention_workspace(n_tokens, heads, kv_heads, maps, dim, vdim, page_size, mask_kind, mask_size);
+    AXK_REQUIRE(partial == nullptr || partial_floats >= need, "masked_attention: a workspace of %ld floats, %ld needed",
+                partial_floats, need);
+    if (need == 0) partial = nullptr;
 #define MA_LAUNCH(MAPS, DT, KC)                                                                                                 \
-  launch_masked_mfma<MAPS, DT, KC>(q, cache, block_table, table_stride, positions, seq_rows, gate, gate_stride, out, tiles, nt, \
+  rc = launch_masked_mfma<MAPS, DT, KC>(q, cache, block_table, table_stride, positions, seq_rows, gate, gate_stride, out, tiles, nt, \
                                    heads, kv_heads, dim, vdim, page_size, mask_kind, mask_size, scale, softcap, lambda,        \
-                                   out_scale, eps, (hipStream_t)stream)
+                                   out_scale, eps, partial, (hipStream_t)stream)
+    int rc = 0;
     if (maps == 1) {
       if (size <= 64) MA_LAUNCH(1, 4, 2); else if (size <= 128) MA_LAUNCH(1, 8, 4); else MA_LAUNCH(1, 16, 8);
     } else {
       if (size <= 64) MA_LAUNCH(2, 4, 2); else if (size <= 128) MA_LAUNCH(2, 8, 4); else MA_LAUNCH(2, 16, 8);
     }
 #undef MA_LAUNCH
+    if (rc != 0) return rc;
     AXK_LAUNCH_CHECK("masked_attention");
     return 0;
   }

@@ -102,7 +102,7 @@ _SIGNATURES = {
     "axk_masked_attention_uses_mfma": [c_int, c_int, c_int, c_int, c_int, c_int],
     "axk_masked_attention": [c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_long, c_void_p, c_int, c_int,
                              c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_float, c_float, c_float, c_float,
-                             c_void_p, c_int, c_void_p],
+                             c_void_p, c_int, c_void_p, c_long, c_void_p],
     "axk_concat_round": [c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_void_p],
     "axk_fill_i32": [c_void_p, c_int, c_int, c_void_p],
     "axk_fill_f32": [c_void_p, c_float, c_int, c_void_p],
@@ -155,6 +155,8 @@ class Kernels:
         self.lib.axk_attention_decode_workspace.restype = ctypes.c_long
         self.lib.axk_latent_attention_workspace.argtypes = [c_int, c_int, c_int, c_int, c_int, c_int]
         self.lib.axk_latent_attention_workspace.restype = ctypes.c_long
+        self.lib.axk_masked_attention_workspace.argtypes = [c_int] * 9
+        self.lib.axk_masked_attention_workspace.restype = ctypes.c_long
         self.lib.axk_packed_elems.argtypes = [c_int, c_int]
         self.lib.axk_packed_elems.restype = ctypes.c_long
         self.lib.axk_gemm_workspace.argtypes = [c_int, c_int, c_int, c_int]
@@ -936,10 +938,13 @@ class Kernels:
         if tiles is not None:
             self._i32(tiles, "attention tiles")
             n_tiles = tiles.shape[0]
+        need = int(self.lib.axk_masked_attention_workspace(T, heads, kv_heads, maps, dim, vdim, page_size, self.MASKS[mask],
+                                                           int(mask_size)))
+        partial = torch.empty(need, dtype=torch.float32, device=out.device) if need else None
         self._check(self.lib.axk_masked_attention(
             _ptr(q), _ptr(cache), _ptr(block_table), block_table.shape[-1], _ptr(positions), _ptr(seq_rows), _ptr(gate),
             gate_stride, _ptr(out), T, heads, kv_heads, maps, dim, vdim, page_size, self.MASKS[mask], int(mask_size), float(scale),
-            float(softcap), float(lam), float(out_scale), float(eps), _ptr(tiles), n_tiles, _stream()))
+            float(softcap), float(lam), float(out_scale), float(eps), _ptr(tiles), n_tiles, _ptr(partial), need, _stream()))
         return out
 
     def fill_i32(self, dst: torch.Tensor, value: int) -> None:

@@ -108,27 +108,49 @@ def _qwen_sizes(width, heads, kv_heads, ff):
                 max_position_embeddings=8192, rope_theta=10000.0, rms_norm_eps=1e-6, tie_word_embeddings=False)
 
 
+# --design figalorn: four layer runs as the dense decoder has layers: a windowed layer whose values are its keys, run
+# twice over (each pass begins with the rewrite of the stream), then two differential layers in chunks; query heads of
+# 128 (two maps of 64 in the differential layers, values of 128), and a two-matrix feed-forward of 1.5 times the gated
+# one's width (the same weights and work a token).
+def _figalorn_sizes(width, heads, kv_heads, ff, window, chunk):
+    keyed = {"type": "attention_2", "mixer": {
+        "heads": heads, "kv_heads": kv_heads, "dim": 128, "vdim": 128, "mask": {"size": window}, "softcap": 30.0,
+        "scale": 128 ** -0.5, "rot": {"base": 10000.0, "dims": 128,
+                                      "scaling": {"factor": 4.0, "original": 2048, "fast": 32.0, "slow": 1.0}}}}
+    diff = {"type": "attention", "mixer": {
+        "heads": heads // 2, "kv_heads": max(kv_heads // 2, 1), "dim": 64, "vdim": 128, "diff": 0.3, "mask": {"size": chunk},
+        "scale": 64 ** -0.5, "rot": {"base": 10000.0, "dims": 32,
+                                     "scaling": {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 2048}}}}
+    mlp = {"kind": "dense", "ff": ff * 3 // 2}
+    return {"architecture": "Figalorn", "layers": [dict(keyed, mlp=mlp), dict(diff, mlp=mlp), dict(diff, mlp=mlp)],
+            "loop": {"start": 0, "stop": 1, "times": 2}, "norm": {"eps": 1e-6}, "vocab": 32000, "width": width}
+
+
 DESIGN_SIZES = {
-    "2048": (_pikesun_sizes(2048, 2560, 10, 16, 768, 32, 4, 704, 1408, 5632, 1024), _qwen_sizes(2048, 16, 2, 5632)),
-    "4096": (_pikesun_sizes(4096, 5120, 20, 32, 1536, 64, 6, 1408, 2816, 11008, 2048), _qwen_sizes(4096, 32, 8, 11008)),
+    "pikesun": {
+        "2048": (_pikesun_sizes(2048, 2560, 10, 16, 768, 32, 4, 704, 1408, 5632, 1024), _qwen_sizes(2048, 16, 2, 5632)),
+        "4096": (_pikesun_sizes(4096, 5120, 20, 32, 1536, 64, 6, 1408, 2816, 11008, 2048), _qwen_sizes(4096, 32, 8, 11008))},
+    "figalorn": {
+        "2048": (_figalorn_sizes(2048, 16, 2, 5632, 1024, 1536), _qwen_sizes(2048, 16, 2, 5632)),
+        "4096": (_figalorn_sizes(4096, 32, 8, 11008, 2048, 8192), _qwen_sizes(4096, 32, 8, 11008))},
 }
 
 
 def design(args, torch) -> int:
-    """Prefill and decoding of the Pikesun design at sizes that resemble real models' layers, beside the
+    """Prefill and decoding of a design (--design) at sizes that resemble real models' layers, beside the
     dense decoder of equal width: a prompt of --prompt tokens (default 2,048) in one step, decoding at
     --batch (default 8) behind such prompts from graphs, and each kind of step kernel by kernel."""
     import axon_amd
     from axon_amd.engine import StepEntry
     T, batch, steps = args.prompt or 2048, args.batch, args.steps or 64
-    out = {"design": "pikesun", "dtype": args.dtype, "prompt_tokens": T, "batch": batch, "data": "synthetic (random weights)",
+    out = {"design": args.design, "dtype": args.dtype, "prompt_tokens": T, "batch": batch, "data": "synthetic (random weights)",
            "sizes": {}}
     gen = torch.Generator().manual_seed(0)
-    for size, pair in DESIGN_SIZES.items():
+    for size, pair in DESIGN_SIZES[args.design].items():
         if args.design_size and size != args.design_size:
             continue
         row = out["sizes"][size] = {}
-        for label, cfg in zip(("pikesun", "qwen2"), pair):
+        for label, cfg in zip((args.design, "qwen2"), pair):
             llm = axon_amd.load(cfg, dtype=args.dtype, random_seed=0, init_std=0.02, page_size=64,
                                 num_pages=(batch + 1) * (-(-(T + steps + args.warmup + 80) // 64)) + 8, max_seqs=batch + 1,
                                 max_batch_tokens=T, max_seq_len=T + steps + args.warmup + 80)
@@ -175,7 +197,7 @@ def design(args, torch) -> int:
 
 def main() -> int:
     ap = argparse.ArgumentParser()
-    ap.add_argument("--design", default="", choices=["", "pikesun"], help="instead of the headline benchmark: prefill and "
+    ap.add_argument("--design", default="", choices=["", "pikesun", "figalorn"], help="instead of the headline benchmark: prefill and "
                     "decoding of this design at sizes that resemble real models' layers, beside the dense decoder of equal size")
     ap.add_argument("--design-size", default="", help="with --design: only this size (2048 or 4096)")
     ap.add_argument("--gpus", type=int, default=1)
