@@ -185,6 +185,24 @@ typedef __attribute__((ext_vector_type(8))) __bf16 ma_bf16x8;
 typedef __attribute__((ext_vector_type(4))) float ma_f32x4;
 __device__ inline ma_bf16x8 ma_frag(uint4 v) { return __builtin_bit_cast(ma_bf16x8, v); }
 
+// Operands come from memory or from LDS; an LDS pointer says so in its type, so that its reads are LDS
+// instructions with a counter of their own and never wait for the loads from memory that are in flight.
+typedef __attribute__((address_space(3))) bf16_t* ma_lds_ptr;
+typedef const __attribute__((address_space(3))) bf16_t* ma_lds_cptr;
+__device__ inline uint4 ma_load16(const bf16_t* p) { return *reinterpret_cast<const uint4*>(p); }
+__device__ inline uint2 ma_load8(const bf16_t* p) { return *reinterpret_cast<const uint2*>(p); }
+typedef __attribute__((ext_vector_type(4))) unsigned ma_u32x4;
+typedef __attribute__((ext_vector_type(2))) unsigned ma_u32x2;
+__device__ inline uint4 ma_load16(ma_lds_cptr p) {
+  return __builtin_bit_cast(uint4, *(const __attribute__((address_space(3))) ma_u32x4*)p);
+}
+__device__ inline uint2 ma_load8(ma_lds_cptr p) {
+  return __builtin_bit_cast(uint2, *(const __attribute__((address_space(3))) ma_u32x2*)p);
+}
+__device__ inline void ma_store16(ma_lds_ptr p, uint4 v) {
+  *(__attribute__((address_space(3))) ma_u32x4*)p = __builtin_bit_cast(ma_u32x4, v);
+}
+
 // The same attention on the matrix cores: one wave per tile of up to sixteen columns, a block of 64
 // positions at a time.  A tile of several tokens (consecutive positions of one request) is those
 // tokens for one query head; a tile of one token is that token for up to sixteen query heads of
@@ -217,12 +235,16 @@ struct MaState {
 // One block of 64 positions from p0 for a wave's columns.  kbase: the block's first key row of the
 // wave's key/value head, rows kstride apart (a map's keys mp * dim further); vbase: its first value
 // row, rows vstride apart, the block's positions side by side; both already moved to the lane's
-// slice (8 g, 4 g).  qfrag(mp, c): the lane's query operand of map mp, chunk c.
-template <int MAPS, int DT, int KC, class QF>
-__device__ inline void ma_block(MaState<MAPS, DT>& st, const bf16_t* kbase, long kstride, const bf16_t* vbase, long vstride,
-                                QF qfrag, int p0, int my_lo, int my_pos, int dim, int dt_n, float scale, float softcap, int j,
-                                int g) {
+// slice (8 g, 4 g).  qfrag(mp, c): the lane's query operand of map mp, chunk c.  full: every column
+// sees every position of the block (no mask to apply).  The running maximum is kept in units of log2 e.
+template <int MAPS, int DT, int KC, class PTR, class QF>
+__device__ inline void ma_block(MaState<MAPS, DT>& st, PTR kbase, int kstride, PTR vbase, int vstride,
+                                QF qfrag, int p0, int my_lo, int my_pos, bool full, int dim, int dt_n, float scale, float softcap,
+                                int j, int g) {
   const int kc = (dim + 31) / 32;
+  // the bend's constants: 2 log2(e) / c into the exponential; c log2(e) and twice that out of it
+  const float bend_in = softcap > 0.0f ? 2.8853900817779268f / softcap : 0.0f;
+  const float softcap_log2 = softcap * 1.4426950408889634f, bend_out = 2.0f * softcap_log2;
   uint4 pf[MAPS][2];
   float fold[MAPS];
 #pragma unroll
@@ -231,38 +253,55 @@ __device__ inline void ma_block(MaState<MAPS, DT>& st, const bf16_t* kbase, long
 #pragma unroll
     for (int pt = 0; pt < 4; ++pt) {
       s[pt] = ma_f32x4{0.0f, 0.0f, 0.0f, 0.0f};
-      const bf16_t* krow = kbase + (long)(16 * pt + j) * kstride + mp * dim;
+      const PTR krow = kbase + (16 * pt + j) * kstride + mp * dim;
       uint4 kf[KC];
 #pragma unroll
       for (int c = 0; c < KC; ++c)
-        kf[c] = (c < kc && 32 * c + 8 * g < dim) ? *reinterpret_cast<const uint4*>(krow + 32 * c) : make_uint4(0u, 0u, 0u, 0u);
+        kf[c] = (c < kc && 32 * c + 8 * g < dim) ? ma_load16(krow + 32 * c) : make_uint4(0u, 0u, 0u, 0u);
 #pragma unroll
       for (int c = 0; c < KC; ++c)
         if (c < kc) s[pt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ma_frag(kf[c]), ma_frag(qfrag(mp, c)), s[pt], 0, 0, 0);
+    }
+    // scores in units of log2 e, so that a weight is one exp2: s log2(e), bent as c tanh(s / c) =
+    // c (1 - 2 / (1 + e^(2 s / c))) where asked
+#pragma unroll
+    for (int pt = 0; pt < 4; ++pt)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        float v = s[pt][i] * scale;
+        if (softcap > 0.0f) {
+          const float e2 = __builtin_amdgcn_exp2f(fminf(v * bend_in, 120.0f));       // e^(2 s / c), kept finite
+          v = fmaf(-bend_out, __builtin_amdgcn_rcpf(1.0f + e2), softcap_log2);
+        } else {
+          v *= 1.4426950408889634f;
+        }
+        s[pt][i] = v;
+      }
+    if (!full) {
+#pragma unroll
+      for (int pt = 0; pt < 4; ++pt)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int p = p0 + 16 * pt + 4 * g + i;
+          s[pt][i] = (p >= my_lo && p <= my_pos) ? s[pt][i] : -INFINITY;
+        }
     }
     float mx = -INFINITY;
 #pragma unroll
     for (int pt = 0; pt < 4; ++pt)
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int p = p0 + 16 * pt + 4 * g + i;
-        float v = s[pt][i] * scale;
-        if (softcap > 0.0f) v = softcap * tanhf(v / softcap);
-        v = (p >= my_lo && p <= my_pos) ? v : -INFINITY;
-        s[pt][i] = v;
-        mx = fmaxf(mx, v);
-      }
+      for (int i = 0; i < 4; ++i) mx = fmaxf(mx, s[pt][i]);
     mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
     mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
     const float m_new = fmaxf(st.m[mp], mx);
     const float m_safe = m_new == -INFINITY ? 0.0f : m_new;      // a column that has seen nothing yet
-    fold[mp] = expf(st.m[mp] - m_safe);
+    fold[mp] = __builtin_amdgcn_exp2f(st.m[mp] - m_safe);
     float sum = 0.0f;
 #pragma unroll
     for (int pt = 0; pt < 4; ++pt)
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        const float w = expf(s[pt][i] - m_safe);        // 0 where the position is not seen
+        const float w = __builtin_amdgcn_exp2f(s[pt][i] - m_safe);        // 0 where the position is not seen
         s[pt][i] = w;
         sum += w;
       }
@@ -282,11 +321,11 @@ __device__ inline void ma_block(MaState<MAPS, DT>& st, const bf16_t* kbase, long
 #pragma unroll
     for (int e = 0; e < VB; ++e) {
       if (d0 + e < dt_n) {
-        const bf16_t* vrow = vbase + (long)(16 * (d0 + e) + j) * vstride;
+        const PTR vrow = vbase + (16 * (d0 + e) + j) * vstride;
 #pragma unroll
         for (int c = 0; c < 2; ++c) {
-          v[e][2 * c] = *reinterpret_cast<const uint2*>(vrow + 32 * c);
-          v[e][2 * c + 1] = *reinterpret_cast<const uint2*>(vrow + 32 * c + 16);
+          v[e][2 * c] = ma_load8(vrow + 32 * c);
+          v[e][2 * c + 1] = ma_load8(vrow + 32 * c + 16);
         }
       }
     }
@@ -397,7 +436,7 @@ masked_attention_mfma_kernel(const bf16_t* __restrict__ q, const bf16_t* __restr
   const int my_pos = my_col ? positions[my_tok] : -1;
   const int my_lo = my_col ? first_seen(my_pos, mask_kind, mask_size) : 0;
   const int pos_first = positions[t0], pos_last = pos_first + n - 1;
-  const int lo_first = first_seen(pos_first, mask_kind, mask_size);
+  const int lo_first = first_seen(pos_first, mask_kind, mask_size), lo_last = first_seen(pos_last, mask_kind, mask_size);
   const int32_t* pages = block_table + (long)seq_rows[t0] * table_stride;
   const int kw = kv_heads * MAPS * dim, dt_n = vdim / 16;
   const long page_elems = (long)page_size * (kw + kv_heads * vdim);
@@ -412,9 +451,9 @@ masked_attention_mfma_kernel(const bf16_t* __restrict__ q, const bf16_t* __restr
   for (int b = b_first; b <= b_last; ++b) {
     const int p0 = b * 64, in0 = p0 % page_size;
     const bf16_t* page = cache + (long)pages[p0 / page_size] * page_elems;
-    ma_block<MAPS, DT, KC>(st, page + (long)in0 * kw + (long)gk * MAPS * dim + 8 * g, kw,
+    ma_block<MAPS, DT, KC, const bf16_t*>(st, page + (long)in0 * kw + (long)gk * MAPS * dim + 8 * g, kw,
                            page + (long)page_size * kw + (long)gk * vdim * page_size + in0 + 4 * g, page_size, qfrag, p0, my_lo,
-                           my_pos, dim, dt_n, scale, softcap, j, g);
+                           my_pos, ncols == 16 && p0 >= lo_last && p0 + 63 <= pos_first, dim, dt_n, scale, softcap, j, g);
   }
   if (split) {
     if (!my_col) return;
@@ -455,21 +494,30 @@ masked_attention_fold_kernel(const float* __restrict__ partial, int n_chunks, co
   for (int mp = 0; mp < MAPS; ++mp) {
     const float* src = partial + (((long)t * heads + h) * n_chunks * MAPS + mp) * (vdim + 2);
     const long step = (long)MAPS * (vdim + 2);
+    // the blocks' (m, l) a lane each, 64 at a time; the largest maximum first, then weights handed round by lane
     float M = -INFINITY;
-    for (int c = 0; c < n_chunks; ++c)
-      if (src[c * step + vdim + 1] > 0.0f) M = fmaxf(M, src[c * step + vdim]);
+    for (int c0 = 0; c0 < n_chunks; c0 += 64) {
+      const int c = c0 + lane;
+      if (c < n_chunks && src[c * step + vdim + 1] > 0.0f) M = fmaxf(M, src[c * step + vdim]);
+    }
+    M = wave_max(M);
     float L = 0.0f, acc[MA_OWN];
 #pragma unroll
     for (int i = 0; i < MA_OWN; ++i) acc[i] = 0.0f;
-    for (int c = 0; c < n_chunks; ++c) {
-      const float lc = src[c * step + vdim + 1];
-      if (!(lc > 0.0f)) continue;
-      const float w = expf(src[c * step + vdim] - M);
-      L = fmaf(w, lc, L);
+    for (int c0 = 0; c0 < n_chunks; c0 += 64) {
+      const int c = c0 + lane;
+      const float lc = c < n_chunks ? src[c * step + vdim + 1] : 0.0f;
+      const float w = lc > 0.0f ? exp2f(src[c * step + vdim] - M) : 0.0f;      // the blocks' maxima are in units of log2 e
+      L += wave_sum(w * lc);
+      const int n_here = min(64, n_chunks - c0);
+#pragma unroll 8
+      for (int k = 0; k < n_here; ++k) {
+        const float wk = __shfl(w, k, 64);
 #pragma unroll
-      for (int i = 0; i < MA_OWN; ++i) {
-        const int d = lane + 64 * i;
-        if (d < vdim) acc[i] = fmaf(w, src[c * step + d], acc[i]);
+        for (int i = 0; i < MA_OWN; ++i) {
+          const int d = lane + 64 * i;
+          if (d < vdim) acc[i] = fmaf(wk, src[(c0 + k) * step + d], acc[i]);
+        }
       }
     }
     const float inv = 1.0f / L;
@@ -542,32 +590,53 @@ masked_attention_staged_kernel(const bf16_t* __restrict__ q, const bf16_t* __res
   const int my_pos = my_col ? positions[my_tok] : -1;
   const int my_lo = my_col ? first_seen(my_pos, mask_kind, mask_size) : 0;
   const int pos_first = positions[t0], pos_last = pos_first + n - 1;
-  const int lo_first = first_seen(pos_first, mask_kind, mask_size);
+  const int lo_first = first_seen(pos_first, mask_kind, mask_size), lo_last = first_seen(pos_last, mask_kind, mask_size);
   const int32_t* pages = block_table + (long)seq_rows[t0] * table_stride;
   const int kw = kv_heads * MAPS * dim, dt_n = vdim / 16;
   const long page_elems = (long)page_size * (kw + kv_heads * vdim);
   const int krow = qw + 8, vrow = 64 + 8, k_pieces = qw / 8;
-  bf16_t* ks = stage;
-  bf16_t* vs = stage + 64 * krow;
+  const ma_lds_ptr ks = (ma_lds_ptr)stage, vs = ks + 64 * krow;
   MaState<MAPS, DT> st;
   st.clear();
-  for (int b = lo_first / 64; b <= pos_last / 64; ++b) {
+  // a block's keys and values travel through registers: asked for while the block before is worked on
+  constexpr int KP = MAPS * KC, VP = (DT + 1) / 2;      // 16-byte pieces a thread brings: 64 rows of keys, vdim rows of values
+  uint4 kreg[KP], vreg[VP];
+  auto fetch = [&](int b) {
     const int p0 = b * 64, in0 = p0 % page_size;
     const bf16_t* page = cache + (long)pages[p0 / page_size] * page_elems;
     const bf16_t* ksrc = page + (long)in0 * kw + (long)gk * qw;
     const bf16_t* vsrc = page + (long)page_size * kw + (long)gk * vdim * page_size + in0;
-    __syncthreads();                                    // the block before has been read
-    for (int idx = threadIdx.x; idx < 64 * k_pieces; idx += MAS_WAVES * 64) {
-      const int r = idx / k_pieces, piece = idx % k_pieces;
-      *reinterpret_cast<uint4*>(ks + r * krow + 8 * piece) = *reinterpret_cast<const uint4*>(ksrc + (long)r * kw + 8 * piece);
+#pragma unroll
+    for (int i = 0; i < KP; ++i) {
+      const int idx = threadIdx.x + MAS_WAVES * 64 * i;
+      if (idx < 64 * k_pieces) kreg[i] = *reinterpret_cast<const uint4*>(ksrc + (long)(idx / k_pieces) * kw + 8 * (idx % k_pieces));
     }
-    for (int idx = threadIdx.x; idx < vdim * 8; idx += MAS_WAVES * 64) {
-      const int r = idx >> 3, piece = idx & 7;
-      *reinterpret_cast<uint4*>(vs + r * vrow + 8 * piece) = *reinterpret_cast<const uint4*>(vsrc + (long)r * page_size + 8 * piece);
+#pragma unroll
+    for (int i = 0; i < VP; ++i) {
+      const int idx = threadIdx.x + MAS_WAVES * 64 * i;
+      if (idx < vdim * 8) vreg[i] = *reinterpret_cast<const uint4*>(vsrc + (long)(idx >> 3) * page_size + 8 * (idx & 7));
+    }
+  };
+  const int b_last = pos_last / 64;
+  fetch(lo_first / 64);
+  for (int b = lo_first / 64; b <= b_last; ++b) {
+    __syncthreads();                                    // the block before has been read
+#pragma unroll
+    for (int i = 0; i < KP; ++i) {
+      const int idx = threadIdx.x + MAS_WAVES * 64 * i;
+      if (idx < 64 * k_pieces) ma_store16(ks + (idx / k_pieces) * krow + 8 * (idx % k_pieces), kreg[i]);
+    }
+#pragma unroll
+    for (int i = 0; i < VP; ++i) {
+      const int idx = threadIdx.x + MAS_WAVES * 64 * i;
+      if (idx < vdim * 8) ma_store16(vs + (idx >> 3) * vrow + 8 * (idx & 7), vreg[i]);
     }
     __syncthreads();
+    if (b < b_last) fetch(b + 1);
+    const int p0 = b * 64;
     if (active)
-      ma_block<MAPS, DT, KC>(st, ks + 8 * g, krow, vs + 4 * g, vrow, qfrag, p0, my_lo, my_pos, dim, dt_n, scale, softcap, j, g);
+      ma_block<MAPS, DT, KC, ma_lds_cptr>(st, ks + 8 * g, krow, vs + 4 * g, vrow, qfrag, p0, my_lo, my_pos,
+                             ncols == 16 && p0 >= lo_last && p0 + 63 <= pos_first, dim, dt_n, scale, softcap, j, g);
   }
   if (active)
     ma_finish<MAPS, DT>(st, my_col, my_tok, my_head, heads, vdim, dt_n, gate, gate_stride, out, lambda, out_scale, eps, g);
