@@ -509,20 +509,30 @@ masked_attention_fold_kernel(const float* __restrict__ partial, int n_chunks, co
       const float lc = c < n_chunks ? src[c * step + vdim + 1] : 0.0f;
       const float w = lc > 0.0f ? exp2f(src[c * step + vdim] - M) : 0.0f;      // the blocks' maxima are in units of log2 e
       L += wave_sum(w * lc);
+      // eight blocks' rows asked for together (a row beyond the last is the last again and weighs nothing)
       const int n_here = min(64, n_chunks - c0);
-#pragma unroll 8
-      for (int k = 0; k < n_here; ++k) {
-        const float wk = __shfl(w, k, 64);
+      for (int k0 = 0; k0 < n_here; k0 += 8) {
+        float rows[8][MA_OWN];
 #pragma unroll
-        for (int i = 0; i < MA_OWN; ++i) {
-          const int d = lane + 64 * i;
-          if (d < vdim) acc[i] = fmaf(wk, src[(c0 + k) * step + d], acc[i]);
+        for (int k = 0; k < 8; ++k) {
+          const float* row = src + (c0 + min(k0 + k, n_here - 1)) * step;
+#pragma unroll
+          for (int i = 0; i < MA_OWN; ++i) rows[k][i] = row[min(lane + 64 * i, vdim - 1)];
+        }
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {
+          const float wk = k0 + k < n_here ? __shfl(w, k0 + k, 64) : 0.0f;
+#pragma unroll
+          for (int i = 0; i < MA_OWN; ++i) acc[i] = fmaf(wk, rows[k][i], acc[i]);
         }
       }
     }
     const float inv = 1.0f / L;
 #pragma unroll
-    for (int i = 0; i < MA_OWN; ++i) o[i] = mp == 0 ? acc[i] * inv : o[i] - lambda * (acc[i] * inv);
+    for (int i = 0; i < MA_OWN; ++i) {
+      const float a = lane + 64 * i < vdim ? acc[i] * inv : 0.0f;      // places beyond vdim hold copies: they count as 0
+      o[i] = mp == 0 ? a : o[i] - lambda * a;
+    }
   }
   if (MAPS > 1) {
     float ss = 0.0f;
