@@ -36,7 +36,7 @@ from typing import List, Optional
 import torch
 
 from ..config.base import ConfigError
-from ..kernels import MODE_ADD_F32, MODE_STORE_F32
+from ..kernels import MODE_ADD_F32, MODE_STORE_F32, PackedMatrix
 from .base import CacheBinding, CacheSpec, Mixer, TensorDecl, build_part, register_mixer
 
 TILE_TOKENS = 16        # tokens of one request a tile of the matrix-core kernel holds
@@ -141,6 +141,10 @@ class MaskedAttention(Mixer):
             self.position.load(store, rt)
 
     # ------------------------------------------------------------------ the step
+    def finishes_following_norm(self, ctx) -> bool:
+        """In steps of many rows the output projection's last kernel also writes the norm behind it."""
+        return isinstance(self.w_o, PackedMatrix) and ctx.rt.k.gemm_then_norm_ok(ctx.n_tokens, self.hidden, self.o_width)
+
     def forward(self, ctx, binding: CacheBinding, h, residual, following=None) -> None:
         k, T = ctx.rt.k, h.shape[0]
         group = ctx.cache.group(binding.group)
@@ -162,7 +166,8 @@ class MaskedAttention(Mixer):
         k.masked_attention(q, cache, group.block_table, ctx.positions, ctx.seq_rows, att, self.heads, self.kv_heads, self.maps,
                            self.dim, self.vdim, group.page_size, self.mask, self.mask_size, self.scale, self.softcap, self.lam,
                            1.0 - self.diff, self.eps, gate=proj[:, self.g_at:] if self.gate else None, tiles=tiles)
-        k.gemm(att, self.w_o, residual, None, MODE_ADD_F32)
+        k.gemm(att, self.w_o, residual, None, MODE_ADD_F32,
+               following_norm=None if following is None else following.as_argument())
 
 
 register_mixer("masked_attention", MaskedAttention)

@@ -83,12 +83,19 @@ class DenseMLP(FeedForward):
         for name in self.n.values():
             store.forget(name)
 
-    def forward(self, ctx, h, out, accumulate: bool = True) -> None:
+    def finishes_following_norm(self, ctx) -> bool:
+        """In steps of many rows the down projection's last kernel also writes the norm behind it."""
+        return isinstance(self.w_down, PackedMatrix) and ctx.rt.k.gemm_then_norm_ok(ctx.n_tokens, self.hidden, self.ff)
+
+    def forward(self, ctx, h, out, following=None, accumulate: bool = True) -> None:
         k = ctx.rt.k
         act = ctx.ws.take((h.shape[0], self.ff), ctx.rt.dtype)
         k.gemm(h, self.w_up, act, None, MODE_STORE)
         k.activation(act, self.activation)
-        k.gemm(act, self.w_down, out, None, MODE_ADD_F32 if accumulate else MODE_STORE_F32)
+        if following is not None and accumulate:
+            k.gemm(act, self.w_down, out, None, MODE_ADD_F32, following_norm=following.as_argument())
+        else:
+            k.gemm(act, self.w_down, out, None, MODE_ADD_F32 if accumulate else MODE_STORE_F32)
 
 
 class ClampedGLUMLP(FeedForward):
