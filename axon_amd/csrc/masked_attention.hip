@@ -92,7 +92,7 @@ heads_prepare_kernel(const float* __restrict__ proj, long stride, int q_at, int 
 // (m, l, o) are rescaled block by block; lane d owns value dims d, d + 64, ...  Then the maps are
 // combined, normed and gated, and the head's vdim outputs stored.
 #define MA_WAVES 4
-#define MA_OWN 4      // value dims a lane owns: vdim up to 256
+#define MA_OWN 8      // value dims a lane owns: vdim up to 512
 __global__ void __launch_bounds__(MA_WAVES * 64)
 masked_attention_kernel(const elem_t* __restrict__ q, const elem_t* __restrict__ cache, const int32_t* __restrict__ block_table,
                         int table_stride, const int32_t* __restrict__ positions, const int32_t* __restrict__ seq_rows,
@@ -611,36 +611,42 @@ masked_attention_staged_kernel(const bf16_t* __restrict__ q, const bf16_t* __res
   // a block's keys and values travel through registers: asked for while the block before is worked on
   constexpr int KP = MAPS * KC, VP = (DT + 1) / 2;      // 16-byte pieces a thread brings: 64 rows of keys, vdim rows of values
   uint4 kreg[KP], vreg[VP];
+  // where a thread's pieces lie in a page and in the stage: the same for every block (-1: none)
+  int k_from[KP], k_to[KP], v_from[VP], v_to[VP];
+#pragma unroll
+  for (int i = 0; i < KP; ++i) {
+    const int idx = threadIdx.x + MAS_WAVES * 64 * i, r = idx / k_pieces, piece = idx % k_pieces;
+    k_from[i] = idx < 64 * k_pieces ? r * kw + 8 * piece : -1;
+    k_to[i] = r * krow + 8 * piece;
+  }
+#pragma unroll
+  for (int i = 0; i < VP; ++i) {
+    const int idx = threadIdx.x + MAS_WAVES * 64 * i;
+    v_from[i] = idx < vdim * 8 ? (idx >> 3) * page_size + 8 * (idx & 7) : -1;
+    v_to[i] = (idx >> 3) * vrow + 8 * (idx & 7);
+  }
   auto fetch = [&](int b) {
     const int p0 = b * 64, in0 = p0 % page_size;
     const bf16_t* page = cache + (long)pages[p0 / page_size] * page_elems;
     const bf16_t* ksrc = page + (long)in0 * kw + (long)gk * qw;
     const bf16_t* vsrc = page + (long)page_size * kw + (long)gk * vdim * page_size + in0;
 #pragma unroll
-    for (int i = 0; i < KP; ++i) {
-      const int idx = threadIdx.x + MAS_WAVES * 64 * i;
-      if (idx < 64 * k_pieces) kreg[i] = *reinterpret_cast<const uint4*>(ksrc + (long)(idx / k_pieces) * kw + 8 * (idx % k_pieces));
-    }
+    for (int i = 0; i < KP; ++i)
+      if (k_from[i] >= 0) kreg[i] = *reinterpret_cast<const uint4*>(ksrc + k_from[i]);
 #pragma unroll
-    for (int i = 0; i < VP; ++i) {
-      const int idx = threadIdx.x + MAS_WAVES * 64 * i;
-      if (idx < vdim * 8) vreg[i] = *reinterpret_cast<const uint4*>(vsrc + (long)(idx >> 3) * page_size + 8 * (idx & 7));
-    }
+    for (int i = 0; i < VP; ++i)
+      if (v_from[i] >= 0) vreg[i] = *reinterpret_cast<const uint4*>(vsrc + v_from[i]);
   };
   const int b_last = pos_last / 64;
   fetch(lo_first / 64);
   for (int b = lo_first / 64; b <= b_last; ++b) {
     __syncthreads();                                    // the block before has been read
 #pragma unroll
-    for (int i = 0; i < KP; ++i) {
-      const int idx = threadIdx.x + MAS_WAVES * 64 * i;
-      if (idx < 64 * k_pieces) ma_store16(ks + (idx / k_pieces) * krow + 8 * (idx % k_pieces), kreg[i]);
-    }
+    for (int i = 0; i < KP; ++i)
+      if (k_from[i] >= 0) ma_store16(ks + k_to[i], kreg[i]);
 #pragma unroll
-    for (int i = 0; i < VP; ++i) {
-      const int idx = threadIdx.x + MAS_WAVES * 64 * i;
-      if (idx < vdim * 8) ma_store16(vs + (idx >> 3) * vrow + 8 * (idx & 7), vreg[i]);
-    }
+    for (int i = 0; i < VP; ++i)
+      if (v_from[i] >= 0) ma_store16(vs + v_to[i], vreg[i]);
     __syncthreads();
     if (b < b_last) fetch(b + 1);
     const int p0 = b * 64;

@@ -42,18 +42,35 @@ from .base import CacheBinding, CacheSpec, Mixer, TensorDecl, build_part, regist
 TILE_TOKENS = 16        # tokens of one request a tile of the matrix-core kernel holds
 
 
-def attention_tiles(ctx) -> Optional[torch.Tensor]:
+def first_seen(pos: int, mask: str, size: int) -> int:
+    """The first position that position `pos` sees under a mask."""
+    if mask == "window":
+        return max(0, pos + 1 - size)
+    if mask == "chunk":
+        return pos // size * size
+    return 0
+
+
+def attention_tiles(ctx, mask: str, size: int) -> Optional[torch.Tensor]:
     """The step's tokens in tiles of up to 16 consecutive tokens of one request, int32 [n, 2] (first
-    token, count) on the device; made once a step.  None in a step of single tokens that may be
-    replayed from a graph: every token is then a tile of its own, which the kernel knows without a list."""
+    token, count) on the device, those that see the most positions first (they run longest, and a
+    kernel ends with its last block); made once a step and mask.  None in a step of single tokens that
+    may be replayed from a graph: every token is then a tile of its own, which the kernel knows without a list."""
     if ctx.decode_only:
         return None
-    tiles = ctx.shared.get("masked_attention_tiles")
+    key = ("masked_attention_tiles", mask, size)
+    tiles = ctx.shared.get(key)
     if tiles is None:
-        rows = [(s.q_start + at, min(TILE_TOKENS, s.q_len - at)) for s in ctx.spans for at in range(0, s.q_len, TILE_TOKENS)]
-        if any(a < 0 or n < 1 or a + n > ctx.n_tokens for a, n in rows):
+        rows = []
+        for s in ctx.spans:
+            for at in range(0, s.q_len, TILE_TOKENS):
+                n = min(TILE_TOKENS, s.q_len - at)
+                first = s.start_pos + at
+                rows.append((first + n - first_seen(first, mask, size), s.q_start + at, n))
+        if any(a < 0 or n < 1 or a + n > ctx.n_tokens for _, a, n in rows):
             raise ValueError("attention tiles: a span lies outside the tokens of the step")
-        tiles = ctx.shared["masked_attention_tiles"] = torch.tensor(rows, dtype=torch.int32).to(ctx.rt.device)
+        rows.sort(key=lambda r: -r[0])
+        tiles = ctx.shared[key] = torch.tensor([(a, n) for _, a, n in rows], dtype=torch.int32).to(ctx.rt.device)
     return tiles
 
 
@@ -81,8 +98,8 @@ class MaskedAttention(Mixer):
             raise ConfigError(f"values that are the keys have their size: vdim {self.vdim}, keys of {self.maps * self.dim}")
         if self.mask not in ("causal", "window", "chunk") or (self.mask != "causal" and self.mask_size < 1):
             raise ConfigError(f"mask {mask!r} is not causal, a window or chunks of a size")
-        if self.vdim > 256:
-            raise ConfigError(f"values of {self.vdim} dims are more than the attention kernel's 256")
+        if self.vdim > 512:
+            raise ConfigError(f"values of {self.vdim} dims are more than the attention kernel's 512")
         self.position = build_part("position", p["position"]) if p.get("position") is not None else None
         self.rot = self.position.rotary_dim if self.position is not None else 0
         if self.rot > self.dim:
@@ -162,7 +179,7 @@ class MaskedAttention(Mixer):
         att = ctx.ws.take((T, self.o_width), ctx.rt.dtype)
         tiles = None
         if k.masked_attention_uses_mfma(self.heads, self.kv_heads, self.maps, self.dim, self.vdim, group.page_size):
-            tiles = attention_tiles(ctx)
+            tiles = attention_tiles(ctx, self.mask, self.mask_size)
         k.masked_attention(q, cache, group.block_table, ctx.positions, ctx.seq_rows, att, self.heads, self.kv_heads, self.maps,
                            self.dim, self.vdim, group.page_size, self.mask, self.mask_size, self.scale, self.softcap, self.lam,
                            1.0 - self.diff, self.eps, gate=proj[:, self.g_at:] if self.gate else None, tiles=tiles)
