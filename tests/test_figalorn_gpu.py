@@ -280,7 +280,8 @@ def test_windowed_attention_whose_values_are_its_keys(entry, width, page, dtype)
     (diff(heads=2, kv_heads=2, dim=40, vdim=144, chunk=64, rot_dims=12, d=0.0), 64, 64),     # chunks of exactly a page
     (diff(heads=20, kv_heads=1, dim=16, vdim=16, chunk=129, rot_dims=16, scaling=None), 96, 128),
     (diff(heads=3, kv_heads=1, dim=6, vdim=10, chunk=7, rot_dims=6, d=0.5), 40, 8),
-    (diff(heads=1, kv_heads=1, dim=10, vdim=4, chunk=1, rot_dims=2), 24, 4)])                # every token a chunk of its own
+    (diff(heads=1, kv_heads=1, dim=10, vdim=4, chunk=1, rot_dims=2), 24, 4),                 # every token a chunk of its own
+    (diff(heads=2, kv_heads=1, dim=8, vdim=320, chunk=30, rot_dims=4), 32, 16)])             # values wider than the matrix cores' tiles
 def test_differential_attention_in_chunks(entry, width, page, dtype):
     check_mixer(entry, width, page, dtype, T=max(2 * entry["mixer"]["mask"]["size"] + 70, 200))
 
