@@ -242,8 +242,8 @@ __device__ inline void ma_block(MaState<MAPS, DT>& st, PTR kbase, int kstride, P
                                 QF qfrag, int p0, int my_lo, int my_pos, bool full, int dim, int dt_n, float scale, float softcap,
                                 int j, int g) {
   const int kc = (dim + 31) / 32;
-  // the bend's constants: 2 log2(e) / c into the exponential; c log2(e) and twice that out of it
-  const float bend_in = softcap > 0.0f ? 2.8853900817779268f / softcap : 0.0f;
+  // the bend's constants: scale 2 log2(e) / c into the exponential; c log2(e) and twice that out of it
+  const float bend_in = softcap > 0.0f ? scale * 2.8853900817779268f / softcap : 0.0f, scale_log2 = scale * 1.4426950408889634f;
   const float softcap_log2 = softcap * 1.4426950408889634f, bend_out = 2.0f * softcap_log2;
   uint4 pf[MAPS][2];
   float fold[MAPS];
@@ -257,7 +257,7 @@ __device__ inline void ma_block(MaState<MAPS, DT>& st, PTR kbase, int kstride, P
       uint4 kf[KC];
 #pragma unroll
       for (int c = 0; c < KC; ++c)
-        kf[c] = (c < kc && 32 * c + 8 * g < dim) ? ma_load16(krow + 32 * c) : make_uint4(0u, 0u, 0u, 0u);
+        if (c < kc) kf[c] = ma_load16(krow + 32 * c);      // beyond dim the query's operand is zero and the row's neighbours are finite
 #pragma unroll
       for (int c = 0; c < KC; ++c)
         if (c < kc) s[pt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ma_frag(kf[c]), ma_frag(qfrag(mp, c)), s[pt], 0, 0, 0);
@@ -268,12 +268,12 @@ __device__ inline void ma_block(MaState<MAPS, DT>& st, PTR kbase, int kstride, P
     for (int pt = 0; pt < 4; ++pt)
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        float v = s[pt][i] * scale;
+        float v;
         if (softcap > 0.0f) {
-          const float e2 = __builtin_amdgcn_exp2f(fminf(v * bend_in, 120.0f));       // e^(2 s / c), kept finite
+          const float e2 = __builtin_amdgcn_exp2f(fminf(s[pt][i] * bend_in, 120.0f));       // e^(2 s / c), kept finite
           v = fmaf(-bend_out, __builtin_amdgcn_rcpf(1.0f + e2), softcap_log2);
         } else {
-          v *= 1.4426950408889634f;
+          v = s[pt][i] * scale_log2;
         }
         s[pt][i] = v;
       }
@@ -637,6 +637,9 @@ masked_attention_staged_kernel(const bf16_t* __restrict__ q, const bf16_t* __res
     for (int i = 0; i < VP; ++i)
       if (v_from[i] >= 0) vreg[i] = *reinterpret_cast<const uint4*>(vsrc + v_from[i]);
   };
+  // the 16 bytes behind each staged key row are read with the last chunk of a map whose dims are no multiple of 32
+  // (against a zero query operand): they hold zeros, never what LDS happened to hold
+  if (threadIdx.x < 64) ma_store16(ks + threadIdx.x * krow + qw, make_uint4(0u, 0u, 0u, 0u));
   const int b_last = pos_last / 64;
   fetch(lo_first / 64);
   for (int b = lo_first / 64; b <= b_last; ++b) {
@@ -671,7 +674,7 @@ static int launch_masked_mfma(const void* q, const void* cache, const int32_t* b
                               float* partial, hipStream_t stream) {
   const int grp = heads / kv_heads;
   const size_t lds = ((size_t)64 * (MAPS * dim + 8) + (size_t)vdim * (64 + 8)) * sizeof(bf16_t);
-  if (tiles != nullptr && partial == nullptr && KC <= 4 && lds <= 64 * 1024) {
+  if (tiles != nullptr && partial == nullptr && KC <= 4 && DT <= 8 && lds <= 64 * 1024) {
     static bool configured = false;
     if (!configured && lds > 48 * 1024) {
       hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&masked_attention_staged_kernel<MAPS, DT, KC>),
@@ -766,7 +769,6 @@ extern "C" int axk_masked_attention(const void* q, const void* cache, const int3
       ((uintptr_t)cache & 15) == 0 && ((uintptr_t)out & 7) == 0) {
     AXK_REQUIRE(tiles == nullptr || n_tiles > 0, "masked_attention: a list of %d tiles", n_tiles);
     const int nt = tiles ? n_tiles : n_tokens;
-    const int size = dim > vdim ? dim : vdim;
     const long need = axk_masked_attention_workspace(n_tokens, heads, kv_heads, maps, dim, vdim, page_size, mask_kind, mask_size);
     AXK_REQUIRE(partial == nullptr || partial_floats >= need, "masked_attention: a workspace of %ld floats, %ld needed",
                 partial_floats, need);
@@ -776,11 +778,18 @@ extern "C" int axk_masked_attention(const void* q, const void* cache, const int3
                                    heads, kv_heads, dim, vdim, page_size, mask_kind, mask_size, scale, softcap, lambda,        \
                                    out_scale, eps, partial, (hipStream_t)stream)
     int rc = 0;
-    if (maps == 1) {
-      if (size <= 64) MA_LAUNCH(1, 4, 2); else if (size <= 128) MA_LAUNCH(1, 8, 4); else MA_LAUNCH(1, 16, 8);
-    } else {
-      if (size <= 64) MA_LAUNCH(2, 4, 2); else if (size <= 128) MA_LAUNCH(2, 8, 4); else MA_LAUNCH(2, 16, 8);
-    }
+    // register tiles by the sizes: chunks of 32 key dims (2, 4 or 8), tiles of 16 value dims (4, 8 or 16)
+#define MA_BY_DIM(MAPS, DT)                                                                  \
+  {                                                                                          \
+    if (dim <= 64) MA_LAUNCH(MAPS, DT, 2); else if (dim <= 128) MA_LAUNCH(MAPS, DT, 4); else MA_LAUNCH(MAPS, DT, 8); \
+  }
+#define MA_BY_VDIM(MAPS)                                                                     \
+  {                                                                                          \
+    if (vdim <= 64) MA_BY_DIM(MAPS, 4) else if (vdim <= 128) MA_BY_DIM(MAPS, 8) else MA_BY_DIM(MAPS, 16) \
+  }
+    if (maps == 1) MA_BY_VDIM(1) else MA_BY_VDIM(2)
+#undef MA_BY_VDIM
+#undef MA_BY_DIM
 #undef MA_LAUNCH
     if (rc != 0) return rc;
     AXK_LAUNCH_CHECK("masked_attention");
